@@ -1,0 +1,107 @@
+"""ctypes binding of libfusedswiglu (the C ABI declared in include/fusedswiglu.h).
+
+The library is built in-tree (fusedswiglu_amd/csrc/libfusedswiglu.so) by `build_library()`
+or `make -C fusedswiglu_amd/csrc`.  There is no CPU fallback: if the library is missing or
+a call fails, the caller gets an exception.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+import threading
+
+_CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
+LIBRARY_PATH = os.path.join(_CSRC, "libfusedswiglu.so")
+
+DTYPE_BF16 = 0
+DTYPE_FP16 = 1
+
+STEP_FORWARD, STEP_INPUT_GRAD, STEP_WEIGHT_GRAD = 0, 1, 2
+
+#: every symbol include/fusedswiglu.h declares
+EXPORTED_SYMBOLS = (
+    "fsw_version",
+    "fsw_status_string",
+    "fsw_last_error",
+    "fsw_uses_tiled_kernel",
+    "fsw_force_edge_kernels",
+    "fsw_swiglu_forward",
+    "fsw_elementwise_backward",
+    "fsw_input_grad",
+    "fsw_weight_grad",
+)
+
+
+class FusedSwiGLUError(RuntimeError):
+    """A libfusedswiglu call returned a non-zero status."""
+
+    def __init__(self, status: int, message: str):
+        super().__init__(f"libfusedswiglu status {status}: {message}")
+        self.status = status
+
+
+class LibraryNotBuiltError(ImportError):
+    """libfusedswiglu.so is missing: the HIP extension was not built."""
+
+
+_lib = None
+_lock = threading.Lock()
+
+
+def build_library(verbose: bool = False, jobs: int = 4) -> str:
+    """Compile the HIP sources for gfx950 with hipcc (works without a GPU) and return the
+    path of the shared library.  Always recompiles."""
+    global _lib
+    cmd = ["make", "-C", _CSRC, f"-j{jobs}", "-B"]
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if verbose or res.returncode != 0:
+        print(res.stdout)
+    if res.returncode != 0:
+        raise RuntimeError("building libfusedswiglu.so failed")
+    _lib = None
+    return LIBRARY_PATH
+
+
+def lib() -> ctypes.CDLL:
+    """The loaded library with argument types set.  Raises LibraryNotBuiltError if absent."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not os.path.exists(LIBRARY_PATH):
+            raise LibraryNotBuiltError(
+                f"{LIBRARY_PATH} not found; build it with `make -C {_CSRC}` "
+                "(or fusedswiglu_amd._abi.build_library()). There is no fallback path."
+            )
+        L = ctypes.CDLL(LIBRARY_PATH)
+        vp, i64, ci = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+        L.fsw_version.restype = ci
+        L.fsw_version.argtypes = []
+        L.fsw_status_string.restype = ctypes.c_char_p
+        L.fsw_status_string.argtypes = [ci]
+        L.fsw_last_error.restype = ctypes.c_char_p
+        L.fsw_last_error.argtypes = []
+        L.fsw_uses_tiled_kernel.restype = ci
+        L.fsw_uses_tiled_kernel.argtypes = [ci, i64, i64, i64, i64, i64, i64, i64, ctypes.c_uint]
+        L.fsw_force_edge_kernels.restype = None
+        L.fsw_force_edge_kernels.argtypes = [ci]
+        L.fsw_swiglu_forward.restype = ci
+        L.fsw_swiglu_forward.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, vp]
+        L.fsw_elementwise_backward.restype = ci
+        L.fsw_elementwise_backward.argtypes = [vp, vp, vp, vp, vp, i64, ci, vp]
+        L.fsw_input_grad.restype = ci
+        L.fsw_input_grad.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, vp]
+        L.fsw_weight_grad.restype = ci
+        L.fsw_weight_grad.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, vp]
+        _lib = L
+    return _lib
+
+
+def check(status: int) -> None:
+    if status != 0:
+        L = lib()
+        msg = L.fsw_last_error().decode() or L.fsw_status_string(status).decode()
+        raise FusedSwiGLUError(status, msg)

@@ -1,0 +1,164 @@
+// extern "C" entry points of libfusedswiglu: argument validation, kernel selection, status codes.
+#include "../../include/fusedswiglu.h"
+#include "fsw_internal.hpp"
+#include <atomic>
+#include <cstdarg>
+#include <cstdio>
+
+namespace {
+
+thread_local char g_err[512] = "";
+std::atomic<int> g_force_edge{0};
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+bool dtype_ok(int d) { return d == FSW_DTYPE_BF16 || d == FSW_DTYPE_FP16; }
+bool al2(const void* p) { return ((uintptr_t)p & 1) == 0; }
+
+int check_dims(const char* fn, int64_t T, int64_t D, int64_t I) {
+  if (T <= 0 || D <= 0 || I <= 0)
+    return fail(FSW_ERR_BAD_SHAPE, "%s: dimensions must be positive (T=%lld D=%lld I=%lld)", fn,
+                (long long)T, (long long)D, (long long)I);
+  if (T > 0x7fffffffLL || D > 0x7fffffffLL || I > 0x7fffffffLL)
+    return fail(FSW_ERR_BAD_SHAPE, "%s: dimension exceeds 2^31-1 (T=%lld D=%lld I=%lld)", fn,
+                (long long)T, (long long)D, (long long)I);
+  return FSW_OK;
+}
+
+int check_ld(const char* fn, const char* name, int64_t ld, int64_t cols) {
+  if (ld < cols)
+    return fail(FSW_ERR_BAD_STRIDE, "%s: leading dimension %s=%lld is smaller than the row length %lld",
+                fn, name, (long long)ld, (long long)cols);
+  return FSW_OK;
+}
+
+int launched(const char* fn, hipError_t e) {
+  if (e != hipSuccess) return fail(FSW_ERR_LAUNCH, "%s: %s", fn, hipGetErrorString(e));
+  return FSW_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int fsw_version(void) { return FSW_VERSION; }
+
+const char* fsw_status_string(int status) {
+  switch (status) {
+    case FSW_OK: return "ok";
+    case FSW_ERR_NULL_POINTER: return "null pointer";
+    case FSW_ERR_BAD_DTYPE: return "unsupported dtype";
+    case FSW_ERR_BAD_SHAPE: return "bad shape";
+    case FSW_ERR_BAD_STRIDE: return "bad leading dimension";
+    case FSW_ERR_ALIGNMENT: return "pointer not 2-byte aligned";
+    case FSW_ERR_LAUNCH: return "kernel launch failed";
+    default: return "unknown status";
+  }
+}
+
+const char* fsw_last_error(void) { return g_err; }
+
+void fsw_force_edge_kernels(int on) { g_force_edge.store(on ? 1 : 0); }
+
+int fsw_uses_tiled_kernel(int step, int64_t T, int64_t D, int64_t I, int64_t ldx, int64_t ldw,
+                          int64_t ldo, int64_t ld_grad, unsigned pointer_alignment) {
+  if (g_force_edge.load()) return 0;
+  // stand-in pointers that carry only the alignment
+  const void* ptr = (const void*)(uintptr_t)(pointer_alignment ? pointer_alignment : 1);
+  fsw::Problem p{};
+  p.x = p.wg = p.wu = p.dG = p.dU = ptr;
+  p.out = p.g = p.u = p.dx = p.dWg = p.dWu = (void*)ptr;
+  p.T = T; p.D = D; p.I = I; p.ldx = ldx; p.ldw = ldw; p.ldo = ldo; p.lddx = ld_grad; p.lddw = ld_grad;
+  switch (step) {
+    case 0: return fsw::fast_path_ok_forward(p) ? 1 : 0;
+    case 1: return fsw::fast_path_ok_input_grad(p) ? 1 : 0;
+    case 2: return fsw::fast_path_ok_weight_grad(p) ? 1 : 0;
+    default: return 0;
+  }
+}
+
+int fsw_swiglu_forward(const void* x, const void* w_gate, const void* w_up, void* out,
+                       void* xw_gate, void* xw_up, int64_t T, int64_t D, int64_t I, int64_t ldx,
+                       int64_t ldw, int64_t ldo, int dtype, void* stream) {
+  const char* fn = "fsw_swiglu_forward";
+  if (!x || !w_gate || !w_up || !out) return fail(FSW_ERR_NULL_POINTER, "%s: x, w_gate, w_up and out must be non-null", fn);
+  if ((xw_gate == nullptr) != (xw_up == nullptr))
+    return fail(FSW_ERR_NULL_POINTER, "%s: xw_gate and xw_up must both be given or both be null", fn);
+  if (!dtype_ok(dtype)) return fail(FSW_ERR_BAD_DTYPE, "%s: dtype %d is neither bf16 (0) nor fp16 (1)", fn, dtype);
+  if (int e = check_dims(fn, T, D, I)) return e;
+  if (int e = check_ld(fn, "ldx", ldx, D)) return e;
+  if (int e = check_ld(fn, "ldw", ldw, I)) return e;
+  if (int e = check_ld(fn, "ldo", ldo, I)) return e;
+  if (!al2(x) || !al2(w_gate) || !al2(w_up) || !al2(out) || !al2(xw_gate) || !al2(xw_up))
+    return fail(FSW_ERR_ALIGNMENT, "%s: pointers must be 2-byte aligned", fn);
+  fsw::Problem p{};
+  p.x = x; p.wg = w_gate; p.wu = w_up; p.out = out; p.g = xw_gate; p.u = xw_up;
+  p.T = T; p.D = D; p.I = I; p.ldx = ldx; p.ldw = ldw; p.ldo = ldo;
+  hipStream_t s = (hipStream_t)stream;
+  if (!g_force_edge.load() && fsw::fast_path_ok_forward(p)) return launched(fn, fsw::launch_forward_fast(dtype, p, s));
+  return launched(fn, fsw::launch_forward_generic(dtype, p, s));
+}
+
+int fsw_elementwise_backward(const void* grad_out, const void* xw_gate, const void* xw_up,
+                             void* grad_xw_up, void* grad_xw_gate, int64_t numel, int dtype,
+                             void* stream) {
+  const char* fn = "fsw_elementwise_backward";
+  if (!grad_out || !xw_gate || !xw_up || !grad_xw_up || !grad_xw_gate)
+    return fail(FSW_ERR_NULL_POINTER, "%s: all five arrays must be non-null", fn);
+  if (!dtype_ok(dtype)) return fail(FSW_ERR_BAD_DTYPE, "%s: dtype %d is neither bf16 (0) nor fp16 (1)", fn, dtype);
+  if (numel <= 0) return fail(FSW_ERR_BAD_SHAPE, "%s: numel must be positive (got %lld)", fn, (long long)numel);
+  if (!al2(grad_out) || !al2(xw_gate) || !al2(xw_up) || !al2(grad_xw_up) || !al2(grad_xw_gate))
+    return fail(FSW_ERR_ALIGNMENT, "%s: pointers must be 2-byte aligned", fn);
+  return launched(fn, fsw::launch_elementwise(dtype, grad_out, xw_gate, xw_up, grad_xw_up, grad_xw_gate,
+                                              (size_t)numel, (hipStream_t)stream));
+}
+
+int fsw_input_grad(const void* grad_xw_gate, const void* grad_xw_up, const void* w_gate,
+                   const void* w_up, void* grad_x, int64_t T, int64_t D, int64_t I, int64_t ldo,
+                   int64_t ldw, int64_t ld_dx, int dtype, void* stream) {
+  const char* fn = "fsw_input_grad";
+  if (!grad_xw_gate || !grad_xw_up || !w_gate || !w_up || !grad_x)
+    return fail(FSW_ERR_NULL_POINTER, "%s: all five arrays must be non-null", fn);
+  if (!dtype_ok(dtype)) return fail(FSW_ERR_BAD_DTYPE, "%s: dtype %d is neither bf16 (0) nor fp16 (1)", fn, dtype);
+  if (int e = check_dims(fn, T, D, I)) return e;
+  if (int e = check_ld(fn, "ldo", ldo, I)) return e;
+  if (int e = check_ld(fn, "ldw", ldw, I)) return e;
+  if (int e = check_ld(fn, "ld_dx", ld_dx, D)) return e;
+  if (!al2(grad_xw_gate) || !al2(grad_xw_up) || !al2(w_gate) || !al2(w_up) || !al2(grad_x))
+    return fail(FSW_ERR_ALIGNMENT, "%s: pointers must be 2-byte aligned", fn);
+  fsw::Problem p{};
+  p.dG = grad_xw_gate; p.dU = grad_xw_up; p.wg = w_gate; p.wu = w_up; p.dx = grad_x;
+  p.T = T; p.D = D; p.I = I; p.ldo = ldo; p.ldw = ldw; p.lddx = ld_dx;
+  hipStream_t s = (hipStream_t)stream;
+  if (!g_force_edge.load() && fsw::fast_path_ok_input_grad(p)) return launched(fn, fsw::launch_input_grad_fast(dtype, p, s));
+  return launched(fn, fsw::launch_input_grad_generic(dtype, p, s));
+}
+
+int fsw_weight_grad(const void* x, const void* grad_xw_up, const void* grad_xw_gate,
+                    void* grad_w_up, void* grad_w_gate, int64_t T, int64_t D, int64_t I,
+                    int64_t ldx, int64_t ldo, int64_t ld_dw, int dtype, void* stream) {
+  const char* fn = "fsw_weight_grad";
+  if (!x || !grad_xw_up || !grad_xw_gate || !grad_w_up || !grad_w_gate)
+    return fail(FSW_ERR_NULL_POINTER, "%s: all five arrays must be non-null", fn);
+  if (!dtype_ok(dtype)) return fail(FSW_ERR_BAD_DTYPE, "%s: dtype %d is neither bf16 (0) nor fp16 (1)", fn, dtype);
+  if (int e = check_dims(fn, T, D, I)) return e;
+  if (int e = check_ld(fn, "ldx", ldx, D)) return e;
+  if (int e = check_ld(fn, "ldo", ldo, I)) return e;
+  if (int e = check_ld(fn, "ld_dw", ld_dw, I)) return e;
+  if (!al2(x) || !al2(grad_xw_up) || !al2(grad_xw_gate) || !al2(grad_w_up) || !al2(grad_w_gate))
+    return fail(FSW_ERR_ALIGNMENT, "%s: pointers must be 2-byte aligned", fn);
+  fsw::Problem p{};
+  p.x = x; p.dG = grad_xw_gate; p.dU = grad_xw_up; p.dWg = grad_w_gate; p.dWu = grad_w_up;
+  p.T = T; p.D = D; p.I = I; p.ldx = ldx; p.ldo = ldo; p.lddw = ld_dw;
+  hipStream_t s = (hipStream_t)stream;
+  if (!g_force_edge.load() && fsw::fast_path_ok_weight_grad(p)) return launched(fn, fsw::launch_weight_grad_fast(dtype, p, s));
+  return launched(fn, fsw::launch_weight_grad_generic(dtype, p, s));
+}
+
+}  // extern "C"

@@ -1,0 +1,136 @@
+// Shared device-side building blocks for the gfx950 (CDNA4) fused SwiGLU kernels:
+// element types, MFMA wrappers, raw buffer descriptors, direct global->LDS loads,
+// LDS swizzles and the XCD-aware tile order.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fsw {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef short i16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+
+#define FSW_LDS __attribute__((address_space(3)))
+#define FSW_DEV __device__ __forceinline__
+
+// ---- element traits -------------------------------------------------------
+struct BF16 {
+  using vec8 = bf16x8;
+  static FSW_DEV f32x16 mfma(i16x8 a, i16x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+  static FSW_DEV float to_float(unsigned short v) { return __uint_as_float((unsigned)v << 16); }
+  // round-to-nearest-even; NaN stays NaN
+  static FSW_DEV unsigned short from_float(float f) {
+    return __builtin_bit_cast(unsigned short, (__bf16)f);
+  }
+};
+struct FP16 {
+  using vec8 = f16x8;
+  static FSW_DEV f32x16 mfma(i16x8 a, i16x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  static FSW_DEV float to_float(unsigned short v) {
+    return (float)__builtin_bit_cast(_Float16, v);
+  }
+  static FSW_DEV unsigned short from_float(float f) {
+    return __builtin_bit_cast(unsigned short, (_Float16)f);
+  }
+};
+
+// silu(g) * u and the gating gradients, fp32 throughout, one rounding at the store.
+FSW_DEV float sigmoidf_fast(float z) { return __frcp_rn(1.0f + __expf(-z)); }
+FSW_DEV float silu_mul(float g, float u) { return g * sigmoidf_fast(g) * u; }
+
+// ---- raw buffer descriptors and direct-to-LDS loads -------------------------
+// Word 3 for gfx90a/gfx94x/gfx950 raw buffers (32-bit data format, no swizzle).
+constexpr int kRsrcWord3 = 0x00020000;
+// A byte offset that is out of range for every descriptor built here (num_records <= 2^31-1):
+// the load then returns zeros, which is how all tile edges are padded.
+constexpr unsigned kOobOffset = 0x80000000u;
+
+FSW_DEV i32x4 make_rsrc(const void* base, unsigned num_records = 0x7fffffffu) {
+  uint64_t a = (uint64_t)base;
+  i32x4 r;
+  r.x = (int)(unsigned)a;
+  r.y = (int)((unsigned)(a >> 32) & 0xffffu);
+  r.z = (int)num_records;
+  r.w = kRsrcWord3;
+  // the descriptor must live in SGPRs
+  r.x = __builtin_amdgcn_readfirstlane(r.x);
+  r.y = __builtin_amdgcn_readfirstlane(r.y);
+  r.z = __builtin_amdgcn_readfirstlane(r.z);
+  return r;
+}
+
+// 16 bytes per lane from `rsrc + voffset` straight into LDS at `lds_addr + lane*16`
+// (the LDS destination of a wave is contiguous by lane; lds_addr is wave-uniform).
+// Counted by vmcnt like any vector load; the compiler does not track it, so every consumer
+// must be fenced with wait_vmcnt<N>() + a workgroup barrier.
+FSW_DEV void load16_to_lds(i32x4 rsrc, unsigned voffset, unsigned lds_addr) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "buffer_load_dwordx4 %1, %2, 0 offen lds"
+      :
+      : "s"(lds_addr), "v"(voffset), "s"(rsrc)
+      : "memory");
+}
+
+template <int N>
+FSW_DEV void wait_vmcnt_and_barrier() {
+  static_assert(N >= 0 && N < 64, "vmcnt is 6 bits");
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "n"(N) : "memory");
+}
+
+// ---- LDS tile formats -------------------------------------------------------
+// Two formats, both for a k-step of BK = 32 elements of a 16-bit type.
+//
+// KC ("k-contiguous"): the operand is row-major with the reduction index innermost.  A tile is
+//   R rows x 64 bytes; the four 16-byte chunks of a row are stored at chunk position
+//   c ^ ((row >> 2) & 3).  Sixteen consecutive rows then cover all 64 LDS banks for a fixed
+//   logical chunk, so the ds_read_b128 fragment reads are conflict free.
+// MC ("m/n-contiguous"): the operand is row-major with the reduction index OUTERMOST.  A panel
+//   is 32 k-rows x 256 bytes (128 columns); the four 64-byte blocks of a row are stored at block
+//   position b ^ (k & 3), so the four k-rows gathered by one ds_read_b64_tr_b16 hit disjoint banks.
+constexpr int kBK = 32;
+constexpr int kKcRowBytes = 64;
+constexpr int kMcRowBytes = 256;
+constexpr int kMcPanelBytes = kBK * kMcRowBytes;  // 8 KiB
+
+// ---- XCD-aware tile order -----------------------------------------------------
+// Workgroups are dealt to the 8 XCDs round-robin by launch index.  Re-number them so that each
+// XCD works through one contiguous range of logical tiles, and inside that range walk bands of
+// `group_m` tile-rows column by column: the ~32 tiles an XCD runs at once then share few A and B
+// panels in that XCD's private L2.
+struct TileCoord {
+  int tm, tn;
+};
+FSW_DEV TileCoord xcd_tile_order(int bid, int tiles_m, int tiles_n, int group_m) {
+  const int nt = tiles_m * tiles_n;
+  const int q = nt >> 3, r = nt & 7;
+  const int xcd = bid & 7, i = bid >> 3;
+  const int lin = (xcd < r) ? xcd * (q + 1) + i : r * (q + 1) + (xcd - r) * q + i;
+  const int per_band = group_m * tiles_n;
+  const int band = lin / per_band;
+  const int first_m = band * group_m;
+  const int rows = min(tiles_m - first_m, group_m);
+  const int in_band = lin - band * per_band;
+  TileCoord t;
+  t.tm = first_m + in_band % rows;
+  t.tn = in_band / rows;
+  return t;
+}
+
+}  // namespace fsw

@@ -1,0 +1,39 @@
+// Host-side declarations shared by the translation units of libfusedswiglu.
+#pragma once
+#include "fsw_common.hpp"
+
+namespace fsw {
+
+// dtype codes used across the library (the C ABI's FSW_DTYPE_* values)
+constexpr int kDtypeBF16 = 0;
+constexpr int kDtypeFP16 = 1;
+
+struct Problem {
+  const void *x, *wg, *wu;       // x [T,D]; Wg, Wu [D,I]
+  const void *dG, *dU;           // [T,I]
+  void *out, *g, *u;             // [T,I]   (g, u may be null in the forward)
+  void *dx;                      // [T,D]
+  void *dWg, *dWu;               // [D,I]
+  long long T, D, I;
+  long long ldx, ldw, ldo;       // leading dimensions (elements) of x, the weights, the [T,I] arrays
+  long long lddx, lddw;          // of dx and of dWg/dWu
+};
+
+// Tiled direct-to-LDS MFMA kernels: need every dimension and leading dimension to be a multiple
+// of 8 elements and every pointer 16-byte aligned.
+bool fast_path_ok_forward(const Problem& p);
+bool fast_path_ok_input_grad(const Problem& p);
+bool fast_path_ok_weight_grad(const Problem& p);
+hipError_t launch_forward_fast(int dtype, const Problem& p, hipStream_t s);
+hipError_t launch_input_grad_fast(int dtype, const Problem& p, hipStream_t s);
+hipError_t launch_weight_grad_fast(int dtype, const Problem& p, hipStream_t s);
+
+// Any shape, any stride, 2-byte alignment: guarded element loads, same MFMA arithmetic.
+hipError_t launch_forward_generic(int dtype, const Problem& p, hipStream_t s);
+hipError_t launch_input_grad_generic(int dtype, const Problem& p, hipStream_t s);
+hipError_t launch_weight_grad_generic(int dtype, const Problem& p, hipStream_t s);
+
+hipError_t launch_elementwise(int dtype, const void* dout, const void* g, const void* u, void* dU,
+                              void* dG, size_t n, hipStream_t stream);
+
+}  // namespace fsw

@@ -1,0 +1,175 @@
+"""dtype-generic host launchers: torch tensors in, raw device pointers through the C ABI.
+
+PyTorch is plumbing here (device memory, the current HIP stream); all arithmetic happens in
+libfusedswiglu.  Mirrors the launcher seam of the reference
+(fused_swiglu/kernels/kernels_bf16.py:162-206, :236-255, :385-412) with these differences:
+  * x may have any number (>= 1) of leading dimensions; they are flattened into T tokens
+    (the reference insists on exactly 3-D input, kernels_bf16.py:178-180);
+  * weight gradients come back already reduced over all tokens, shape [D, I];
+  * the input gradient has its own launcher instead of two torch matmuls (swiglu.py:45).
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from .. import _abi
+
+
+class ShapeError(AssertionError, ValueError):
+    """Bad shape / dtype / device.  The reference signals these with `assert`
+    (kernels_bf16.py:170-182); this is an AssertionError and a ValueError at once."""
+
+
+_DTYPE_CODE = {torch.bfloat16: _abi.DTYPE_BF16, torch.float16: _abi.DTYPE_FP16}
+
+
+def _require(cond: bool, msg: str) -> None:
+    if not cond:
+        raise ShapeError(msg)
+
+
+def _check_device(*tensors: torch.Tensor) -> torch.device:
+    dev = tensors[0].device
+    _require(dev.type == "cuda", f"fused SwiGLU needs tensors on a HIP GPU, got device '{dev}'")
+    for t in tensors[1:]:
+        _require(t.device == dev, f"all tensors must be on the same device ({t.device} vs {dev})")
+    return dev
+
+
+def _stream_ptr(dev: torch.device) -> int:
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+def _rows(t: torch.Tensor) -> torch.Tensor:
+    """2-D [rows, cols] view with unit inner stride (copies only if it must)."""
+    t2 = t.reshape(-1, t.shape[-1])
+    if t2.stride(-1) != 1 or (t2.shape[0] > 1 and t2.stride(0) < t2.shape[1]):
+        t2 = t2.contiguous()
+    return t2
+
+
+def _ld(t2: torch.Tensor) -> int:
+    return t2.stride(0) if t2.shape[0] > 1 else t2.shape[1]
+
+
+def fused_swiglu_fwd(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, dtype: torch.dtype,
+                     save_preactivations: bool = True
+                     ) -> Tuple[torch.Tensor, Optional[torch.Tensor], Optional[torch.Tensor]]:
+    """out = silu(x @ w_gate) * (x @ w_up); returns (out, x@w_gate, x@w_up) like
+    kernels_bf16.py:162-206.  With save_preactivations=False the two pre-activation arrays are
+    neither allocated nor written and None is returned for them."""
+    _require(x.ndim >= 2 and w_up.ndim == 2 and w_gate.ndim == 2,
+             "Incorrect number of dimensions for LHS or RHS")
+    _require(x.shape[-1] == w_up.shape[0],
+             f"Dimension mismatch. Expected x.shape[-1] ({x.shape[-1]}) to be equal to "
+             f"w_up.shape[0] ({w_up.shape[0]})")
+    _require(w_up.shape == w_gate.shape, "Expected both weight matrices to have same shape")
+    _require(x.dtype == dtype and w_gate.dtype == dtype and w_up.dtype == dtype,
+             f"Expected {dtype} inputs and weights, got {x.dtype}, {w_gate.dtype}, {w_up.dtype}")
+    dev = _check_device(x, w_gate, w_up)
+    D, I = w_up.shape
+    _require(x.numel() > 0 and I > 0, "empty input")
+    x2, wg, wu = _rows(x), _rows(w_gate), _rows(w_up)
+    if _ld(wg) != _ld(wu):
+        wg, wu = wg.contiguous(), wu.contiguous()
+    T = x2.shape[0]
+    out_shape = tuple(x.shape[:-1]) + (I,)
+    out = torch.empty(out_shape, device=dev, dtype=dtype)
+    g = torch.empty_like(out) if save_preactivations else None
+    u = torch.empty_like(out) if save_preactivations else None
+    with torch.cuda.device(dev):
+        _abi.check(_abi.lib().fsw_swiglu_forward(
+            x2.data_ptr(), wg.data_ptr(), wu.data_ptr(), out.data_ptr(),
+            g.data_ptr() if g is not None else None, u.data_ptr() if u is not None else None,
+            T, D, I, _ld(x2), _ld(wg), I, _DTYPE_CODE[dtype], _stream_ptr(dev)))
+    return out, g, u
+
+
+def elementwise_backward(grad_output: torch.Tensor, xw_gate: torch.Tensor, xw_up: torch.Tensor,
+                         dtype: torch.dtype) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Returns (grad_xw_up, grad_xw_gate) -- the reference's order (kernels_bf16.py:255)."""
+    _require(grad_output.shape == xw_gate.shape == xw_up.shape,
+             "grad_output, xw_gate and xw_up must have the same shape")
+    _require(grad_output.dtype == dtype and xw_gate.dtype == dtype and xw_up.dtype == dtype,
+             f"Expected {dtype} tensors")
+    dev = _check_device(grad_output, xw_gate, xw_up)
+    _require(grad_output.numel() > 0, "empty input")
+    # the kernel indexes flat, dense arrays (the reference silently assumes this, :224-226)
+    dout, g, u = grad_output.contiguous(), xw_gate.contiguous(), xw_up.contiguous()
+    grad_xw_up = torch.empty_like(dout)
+    grad_xw_gate = torch.empty_like(dout)
+    with torch.cuda.device(dev):
+        _abi.check(_abi.lib().fsw_elementwise_backward(
+            dout.data_ptr(), g.data_ptr(), u.data_ptr(), grad_xw_up.data_ptr(),
+            grad_xw_gate.data_ptr(), dout.numel(), _DTYPE_CODE[dtype], _stream_ptr(dev)))
+    return grad_xw_up, grad_xw_gate
+
+
+def fused_input_grad(grad_xw_gate: torch.Tensor, grad_xw_up: torch.Tensor, w_gate: torch.Tensor,
+                     w_up: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """grad_x = grad_xw_gate @ w_gate.T + grad_xw_up @ w_up.T in one kernel (swiglu.py:45)."""
+    _require(grad_xw_gate.shape == grad_xw_up.shape, "gate/up gradient shapes differ")
+    _require(w_gate.ndim == 2 and w_gate.shape == w_up.shape,
+             "Expected both weight matrices to have same shape")
+    _require(grad_xw_gate.shape[-1] == w_gate.shape[1], "Dimension mismatch between gradients and weights")
+    _require(all(t.dtype == dtype for t in (grad_xw_gate, grad_xw_up, w_gate, w_up)),
+             f"Expected {dtype} tensors")
+    dev = _check_device(grad_xw_gate, grad_xw_up, w_gate, w_up)
+    D, I = w_gate.shape
+    dg, du, wg, wu = _rows(grad_xw_gate), _rows(grad_xw_up), _rows(w_gate), _rows(w_up)
+    if _ld(dg) != _ld(du):
+        dg, du = dg.contiguous(), du.contiguous()
+    if _ld(wg) != _ld(wu):
+        wg, wu = wg.contiguous(), wu.contiguous()
+    T = dg.shape[0]
+    grad_x = torch.empty(tuple(grad_xw_gate.shape[:-1]) + (D,), device=dev, dtype=dtype)
+    with torch.cuda.device(dev):
+        _abi.check(_abi.lib().fsw_input_grad(
+            dg.data_ptr(), du.data_ptr(), wg.data_ptr(), wu.data_ptr(), grad_x.data_ptr(),
+            T, D, I, _ld(dg), _ld(wg), D, _DTYPE_CODE[dtype], _stream_ptr(dev)))
+    return grad_x
+
+
+def fused_weight_grad(x: torch.Tensor, grad_xw_up: torch.Tensor, grad_xw_gate: torch.Tensor,
+                      dtype: torch.dtype) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(grad_w_up, grad_w_gate) = (x^T grad_xw_up, x^T grad_xw_gate), each [D, I], reduced over
+    every token in fp32.  Same argument and return order as fused_bmm (kernels_bf16.py:385-412),
+    with the batch sum of swiglu.py:56-57 folded in."""
+    _require(grad_xw_up.shape == grad_xw_gate.shape, "gate/up gradient shapes differ")
+    _require(x.shape[:-1] == grad_xw_up.shape[:-1],
+             f"Dimension mismatch. x {tuple(x.shape)} vs gradients {tuple(grad_xw_up.shape)}")
+    _require(all(t.dtype == dtype for t in (x, grad_xw_up, grad_xw_gate)), f"Expected {dtype} tensors")
+    dev = _check_device(x, grad_xw_up, grad_xw_gate)
+    x2, du, dg = _rows(x), _rows(grad_xw_up), _rows(grad_xw_gate)
+    if _ld(dg) != _ld(du):
+        dg, du = dg.contiguous(), du.contiguous()
+    T, D = x2.shape
+    I = du.shape[1]
+    grad_w_up = torch.empty((D, I), device=dev, dtype=dtype)
+    grad_w_gate = torch.empty((D, I), device=dev, dtype=dtype)
+    with torch.cuda.device(dev):
+        _abi.check(_abi.lib().fsw_weight_grad(
+            x2.data_ptr(), du.data_ptr(), dg.data_ptr(), grad_w_up.data_ptr(), grad_w_gate.data_ptr(),
+            T, D, I, _ld(x2), _ld(du), I, _DTYPE_CODE[dtype], _stream_ptr(dev)))
+    return grad_w_up, grad_w_gate
+
+
+def fused_bmm(x_t: torch.Tensor, grad_xw_up: torch.Tensor, grad_xw_gate: torch.Tensor,
+              dtype: torch.dtype) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Signature-compatible with the reference's fused_bmm (kernels_bf16.py:385-412):
+    x_t is the [B, D, S] view of x, the gradients are [B, S, I]; returns per-batch
+    (grad_w_up, grad_w_gate) of shape [B, D, I].  The autograd Functions of this package use
+    fused_weight_grad instead, which reduces over the batch inside the kernel."""
+    _require(x_t.ndim == 3 and grad_xw_up.ndim == 3, "Incorrect number of dimensions for LHS or RHS")
+    _require(x_t.shape[-1] == grad_xw_up.shape[-2],
+             f"Dimension mismatch. Expected x.shape[2] ({x_t.shape[-1]}) to be equal to "
+             f"grad.shape[1] ({grad_xw_up.shape[-2]})")
+    B = x_t.shape[0]
+    ups, gates = [], []
+    for b in range(B):
+        gu, gg = fused_weight_grad(x_t[b].transpose(0, 1), grad_xw_up[b], grad_xw_gate[b], dtype)
+        ups.append(gu)
+        gates.append(gg)
+    return torch.stack(ups), torch.stack(gates)

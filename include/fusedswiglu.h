@@ -1,0 +1,110 @@
+/*
+ * libfusedswiglu -- C ABI of the MI355X (gfx950) fused SwiGLU forward/backward.
+ *
+ * This is the drop-in boundary underneath the two autograd Functions of
+ * fattorib/fusedswiglu (`FusedSwiGLU`, fused_swiglu/swiglu.py:16-58, and
+ * `FastAccumFusedSwiGLU`, fused_swiglu/swiglu_f16.py:16-58).  The reference has no
+ * FFI of its own: its seam is the three Python launchers in
+ * fused_swiglu/kernels/kernels_bf16.py (and the fp16 twins in kernels_fp16.py), plus one
+ * line of torch matmuls for the input gradient.  Each entry point below replaces one of
+ * those and is what a ctypes / pybind / cgo binding for this path would bind.
+ *
+ * Conventions
+ *   - T = number of tokens (all leading dimensions of x flattened), D = d_model,
+ *     I = d_intermediate.  All matrices are row-major with unit inner stride; `ld*`
+ *     arguments are leading dimensions (row pitches) in ELEMENTS.
+ *   - Every pointer is a device pointer on the current HIP device.  The caller owns every
+ *     buffer; the library never allocates, frees or keeps a pointer after returning.
+ *   - `dtype` selects 16-bit storage: FSW_DTYPE_BF16 or FSW_DTYPE_FP16.  Products are
+ *     accumulated in fp32 on the MFMA units for both (CDNA4 has no fp16-accumulate mode,
+ *     so the reference's fp16 "fast accumulation" maps to fp32 accumulation).
+ *   - `stream` is a hipStream_t (NULL = the default stream).  Calls only enqueue work; they
+ *     never synchronize.  The library is stateless and re-entrant.
+ *   - Return value: FSW_OK or an FSW_ERR_* code; arguments are validated before anything is
+ *     enqueued.  fsw_last_error() gives a thread-local message for the last failure.
+ *   - Operands whose dimensions and leading dimensions are multiples of 8 elements and whose
+ *     pointers are 16-byte aligned run on the tiled direct-to-LDS MFMA kernels; anything else
+ *     runs on a slower edge-shape kernel with identical arithmetic.
+ */
+#ifndef FUSEDSWIGLU_H_
+#define FUSEDSWIGLU_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FSW_VERSION 100 /* major*10000 + minor*100 + patch */
+
+enum { FSW_DTYPE_BF16 = 0, FSW_DTYPE_FP16 = 1 };
+
+enum {
+  FSW_OK = 0,
+  FSW_ERR_NULL_POINTER = 1,
+  FSW_ERR_BAD_DTYPE = 2,
+  FSW_ERR_BAD_SHAPE = 3,  /* a dimension is <= 0 or exceeds 2^31-1 */
+  FSW_ERR_BAD_STRIDE = 4, /* a leading dimension is smaller than the row it describes */
+  FSW_ERR_ALIGNMENT = 5,  /* a pointer is not 2-byte aligned */
+  FSW_ERR_LAUNCH = 6      /* the HIP runtime refused the launch; see fsw_last_error() */
+};
+
+/* Library version (FSW_VERSION it was built with). */
+int fsw_version(void);
+/* Static description of a status code. */
+const char* fsw_status_string(int status);
+/* Message of the calling thread's most recent failed call ("" if none). */
+const char* fsw_last_error(void);
+/* 1 if the arguments of the named step would run on the tiled kernels, 0 if on the
+ * edge-shape kernel.  step: 0 forward, 1 input_grad, 2 weight_grad.  Pure host logic. */
+int fsw_uses_tiled_kernel(int step, int64_t T, int64_t D, int64_t I, int64_t ldx, int64_t ldw,
+                          int64_t ldo, int64_t ld_grad, unsigned pointer_alignment);
+/* Test hook: nonzero forces every later call of this process onto the edge-shape kernels. */
+void fsw_force_edge_kernels(int on);
+
+/*
+ * Forward: g = x Wg, u = x Wu, out = silu(g) * u.
+ * Replaces fused_swiglu_fwd + swiglu_kernel (fused_swiglu/kernels/kernels_bf16.py:162-206,
+ * :41-160; fp16: kernels_fp16.py:171-216).
+ *   x [T,D] (ldx)   w_gate, w_up [D,I] (ldw)   out, xw_gate, xw_up [T,I] (ldo)
+ * xw_gate and xw_up (the pre-activations the backward needs) may both be NULL, in which
+ * case they are not written (inference).
+ */
+int fsw_swiglu_forward(const void* x, const void* w_gate, const void* w_up, void* out,
+                       void* xw_gate, void* xw_up, int64_t T, int64_t D, int64_t I, int64_t ldx,
+                       int64_t ldw, int64_t ldo, int dtype, void* stream);
+
+/*
+ * Gating gradient: grad_xw_up = grad_out * silu(xw_gate),
+ *                  grad_xw_gate = grad_out * xw_up * silu'(xw_gate).
+ * Replaces elementwise_backward + kernel (kernels_bf16.py:236-255, :210-234).  All five
+ * arrays are dense with `numel` elements.
+ */
+int fsw_elementwise_backward(const void* grad_out, const void* xw_gate, const void* xw_up,
+                             void* grad_xw_up, void* grad_xw_gate, int64_t numel, int dtype,
+                             void* stream);
+
+/*
+ * Input gradient: grad_x = grad_xw_gate Wg^T + grad_xw_up Wu^T, one kernel, one accumulator.
+ * Replaces the two torch matmuls and the add at fused_swiglu/swiglu.py:45.
+ *   grad_xw_gate, grad_xw_up [T,I] (ldo)   w_gate, w_up [D,I] (ldw)   grad_x [T,D] (ld_dx)
+ */
+int fsw_input_grad(const void* grad_xw_gate, const void* grad_xw_up, const void* w_gate,
+                   const void* w_up, void* grad_x, int64_t T, int64_t D, int64_t I, int64_t ldo,
+                   int64_t ldw, int64_t ld_dx, int dtype, void* stream);
+
+/*
+ * Weight gradients: grad_w_gate = x^T grad_xw_gate, grad_w_up = x^T grad_xw_up, reduced over
+ * all T tokens in fp32.  Replaces fused_bmm + bmm_kernel (kernels_bf16.py:385-412, :280-382)
+ * together with the batch sum `unbroadcast` (fused_swiglu/swiglu.py:11-13, :56-57).
+ *   x [T,D] (ldx)   grad_xw_up, grad_xw_gate [T,I] (ldo)   grad_w_up, grad_w_gate [D,I] (ld_dw)
+ * Argument order (up before gate) follows fused_bmm.
+ */
+int fsw_weight_grad(const void* x, const void* grad_xw_up, const void* grad_xw_gate,
+                    void* grad_w_up, void* grad_w_gate, int64_t T, int64_t D, int64_t I,
+                    int64_t ldx, int64_t ldo, int64_t ld_dw, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FUSEDSWIGLU_H_ */

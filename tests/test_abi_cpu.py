@@ -1,0 +1,139 @@
+"""CPU-only checks of the C-ABI library and the host logic: the library loads, exports every
+symbol the header declares, validates its arguments before touching the GPU, and the Python
+boundary raises the reference's kind of errors.  No kernel is launched here."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from fusedswiglu_amd import FastAccumFusedSwiGLU, FusedSwiGLU, _abi
+from fusedswiglu_amd.kernels import kernels_bf16, kernels_fp16
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def L():
+    if not os.path.exists(_abi.LIBRARY_PATH):
+        _abi.build_library()
+    return _abi.lib()
+
+
+def test_header_symbols_all_exported(L):
+    header = open(os.path.join(ROOT, "include", "fusedswiglu.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(fsw_[a-z_0-9]+)\s*\(", header))
+    assert declared == set(_abi.EXPORTED_SYMBOLS)
+    for name in declared:
+        assert getattr(L, name) is not None
+    m = re.search(r"#define FSW_VERSION (\d+)", header)
+    assert L.fsw_version() == int(m.group(1))
+
+
+def test_status_strings(L):
+    assert L.fsw_status_string(0) == b"ok"
+    seen = {L.fsw_status_string(i) for i in range(0, 7)}
+    assert len(seen) == 7
+    assert L.fsw_status_string(99) == b"unknown status"
+
+
+P = ctypes.c_void_p(0x1000)  # a fake, aligned, non-null "device pointer": never dereferenced here
+
+
+def test_forward_validation(L):
+    f = L.fsw_swiglu_forward
+    assert f(None, P, P, P, P, P, 8, 8, 8, 8, 8, 8, 0, None) == 1
+    assert b"non-null" in L.fsw_last_error()
+    assert f(P, P, P, P, P, None, 8, 8, 8, 8, 8, 8, 0, None) == 1  # only one of g/u
+    assert f(P, P, P, P, P, P, 8, 8, 8, 8, 8, 8, 7, None) == 2
+    assert f(P, P, P, P, P, P, 0, 8, 8, 8, 8, 8, 0, None) == 3
+    assert f(P, P, P, P, P, P, 8, -1, 8, 8, 8, 8, 0, None) == 3
+    assert f(P, P, P, P, P, P, 2 ** 31, 8, 8, 8, 8, 8, 0, None) == 3
+    assert f(P, P, P, P, P, P, 8, 8, 8, 7, 8, 8, 0, None) == 4  # ldx < D
+    assert f(P, P, P, P, P, P, 8, 8, 16, 8, 8, 16, 1, None) == 4  # ldw < I
+    assert f(P, P, P, P, P, P, 8, 8, 16, 8, 16, 8, 1, None) == 4  # ldo < I
+    assert f(ctypes.c_void_p(0x1001), P, P, P, P, P, 8, 8, 8, 8, 8, 8, 0, None) == 5
+    assert L.fsw_last_error() != b""
+
+
+def test_backward_validation(L):
+    e = L.fsw_elementwise_backward
+    assert e(P, P, None, P, P, 8, 0, None) == 1
+    assert e(P, P, P, P, P, 0, 0, None) == 3
+    assert e(P, P, P, P, P, 8, 2, None) == 2
+    dx = L.fsw_input_grad
+    assert dx(P, P, P, P, None, 8, 8, 8, 8, 8, 8, 0, None) == 1
+    assert dx(P, P, P, P, P, 8, 8, 8, 8, 8, 4, 0, None) == 4  # ld_dx < D
+    assert dx(P, P, P, P, P, 8, 8, 0, 8, 8, 8, 0, None) == 3
+    dw = L.fsw_weight_grad
+    assert dw(P, None, P, P, P, 8, 8, 8, 8, 8, 8, 1, None) == 1
+    assert dw(P, P, P, P, P, 8, 8, 8, 8, 8, 8, -3, None) == 2
+    assert dw(P, P, P, P, P, 8, 16, 8, 8, 8, 8, 1, None) == 4  # ldx < D
+
+
+def test_kernel_selection_logic(L):
+    t = L.fsw_uses_tiled_kernel
+    # the north-star shape and the fp16 config run on the tiled kernels in all three steps
+    for step in range(3):
+        assert t(step, 8192, 4096, 12288, 4096, 12288, 12288, 4096 if step == 1 else 12288, 16) == 1
+        assert t(step, 8192, 4096, 11008, 4096, 11008, 11008, 4096 if step == 1 else 11008, 16) == 1
+    # dimensions that are not multiples of 8, or unaligned pointers, take the edge-shape kernel
+    assert t(0, 8192, 4096, 11007, 4096, 11007, 11007, 11007, 16) == 0
+    assert t(0, 8192, 4100, 12288, 4100, 12288, 12288, 12288, 16) == 0
+    assert t(0, 8192, 4096, 12288, 4096, 12288, 12288, 12288, 2) == 0
+    # the token count is free: it is never the contiguous index of an operand
+    assert t(0, 8191, 4096, 12288, 4096, 12288, 12288, 12288, 16) == 1
+    assert t(2, 8191, 4096, 12288, 4096, 12288, 12288, 12288, 16) == 1
+    L.fsw_force_edge_kernels(1)
+    try:
+        assert t(0, 8192, 4096, 12288, 4096, 12288, 12288, 12288, 16) == 0
+    finally:
+        L.fsw_force_edge_kernels(0)
+    assert t(0, 8192, 4096, 12288, 4096, 12288, 12288, 12288, 16) == 1
+
+
+def test_python_boundary_errors_without_gpu():
+    """Shape / dtype / device problems raise before any launch, as AssertionError like the
+    reference's asserts (fused_swiglu/kernels/kernels_bf16.py:170-182) and as ValueError."""
+    bf = torch.bfloat16
+    x = torch.zeros(2, 4, 8, dtype=bf)
+    w = torch.zeros(8, 16, dtype=bf)
+    with pytest.raises(AssertionError, match="Dimension mismatch"):
+        kernels_bf16.fused_swiglu_fwd(x, torch.zeros(9, 16, dtype=bf), torch.zeros(9, 16, dtype=bf))
+    with pytest.raises(ValueError, match="same shape"):
+        kernels_bf16.fused_swiglu_fwd(x, w, torch.zeros(8, 24, dtype=bf))
+    with pytest.raises(AssertionError, match="number of dimensions"):
+        kernels_bf16.fused_swiglu_fwd(x, w[None], w[None])
+    with pytest.raises(AssertionError, match="bfloat16"):
+        kernels_bf16.fused_swiglu_fwd(x.float(), w.float(), w.float())
+    with pytest.raises(AssertionError, match="float16"):
+        kernels_fp16.fused_swiglu_fwd(x, w, w)
+    # right shapes and dtype but host tensors: refused, never computed on the CPU
+    with pytest.raises(AssertionError, match="HIP GPU"):
+        kernels_bf16.fused_swiglu_fwd(x, w, w)
+    with pytest.raises(AssertionError, match="HIP GPU"):
+        FusedSwiGLU.apply(x, w, w)
+    with pytest.raises(AssertionError, match="HIP GPU"):
+        FastAccumFusedSwiGLU.apply(x.half().requires_grad_(), w.half(), w.half())
+    with pytest.raises(AssertionError, match="same shape"):
+        kernels_bf16.elementwise_backward(torch.zeros(2, 3, dtype=bf), torch.zeros(2, 4, dtype=bf), torch.zeros(2, 3, dtype=bf))
+
+
+def test_package_exports():
+    import fusedswiglu_amd
+
+    assert fusedswiglu_amd.__all__ == ["FusedSwiGLU", "FastAccumFusedSwiGLU"]
+    assert issubclass(FusedSwiGLU, torch.autograd.Function)
+    assert issubclass(FastAccumFusedSwiGLU, torch.autograd.Function)
+
+
+def test_product_does_not_import_oracle():
+    """The oracle is test infrastructure: nothing under the package may reference it."""
+    pkg = os.path.join(ROOT, "fusedswiglu_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for fn in files:
+            if fn.endswith((".py", ".hip", ".hpp", ".h", "Makefile")):
+                text = open(os.path.join(dirpath, fn)).read()
+                assert "oracle" not in text.lower(), f"{fn} mentions the oracle"
