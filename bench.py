@@ -1,0 +1,219 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused SwiGLU forward+backward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one `FusedSwiGLU.apply(x, Wg, Wu)` forward plus `out.backward(dout)` on synthetic,
+HBM-resident bf16 inputs of the headline configuration (x [4,2048,4096], Wg/Wu [4096,12288],
+all ~N(0,1) resp. N(0,1/D), seed 0).  Prints ONE JSON line: whole-step TFLOP/s (12*T*D*I flop per
+step), a roofline object for the dominant kernel measured live with GPU events on the launch
+stream, and the eager fp32 PyTorch SwiGLU timed on this machine's host cores as CPU baseline.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16/fp16 MFMA
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra", action="store_true", help="skip the skinny-M and per-kernel extras")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run three plain 1 GiB device copies (known HBM traffic) so that profiler "
+                         "byte counters collected over this run can be scaled")
+    return ap.parse_args()
+
+
+def gpu_time_ms(fn, iters, warmup=3):
+    """Average GPU duration of fn() over `iters` back-to-back launches, from events recorded on
+    the stream the kernels are launched on (torch's current stream)."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    e1.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus must be 1 (multi-GPU sharding is "
+              "described in DESIGN.md, not implemented)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from fusedswiglu_amd import FusedSwiGLU, _abi
+
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    L = _abi.lib()  # raises if the HIP library is not built: no fallback
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    dt = torch.bfloat16
+    B, S, D, I = 4, 2048, 4096, 12288
+    T = B * S
+    x = torch.randn(B, S, D, device=dev, dtype=torch.float32).to(dt).requires_grad_(True)
+    wg = (torch.randn(D, I, device=dev, dtype=torch.float32) / D ** 0.5).to(dt).requires_grad_(True)
+    wu = (torch.randn(D, I, device=dev, dtype=torch.float32) / D ** 0.5).to(dt).requires_grad_(True)
+    dout = torch.randn(B, S, I, device=dev, dtype=torch.float32).to(dt)
+
+    def step():
+        x.grad = wg.grad = wu.grad = None
+        out = FusedSwiGLU.apply(x, wg, wu)
+        out.backward(dout)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt_s = time.perf_counter() - t0
+    ms_per_step = dt_s * 1e3 / args.steps
+    flop_step = 12.0 * T * D * I
+    tflops = flop_step / (ms_per_step * 1e-3) / 1e12
+
+    # ---- per-kernel durations through the C ABI (pre-allocated buffers, launch stream events)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    xd, wgd, wud = x.detach(), wg.detach(), wu.detach()
+    out = torch.empty(B, S, I, device=dev, dtype=dt)
+    g, u = torch.empty_like(out), torch.empty_like(out)
+    dG, dU = torch.empty_like(out), torch.empty_like(out)
+    dx = torch.empty(B, S, D, device=dev, dtype=dt)
+    dWg, dWu = torch.empty(D, I, device=dev, dtype=dt), torch.empty(D, I, device=dev, dtype=dt)
+    p = lambda t: t.data_ptr()  # noqa: E731
+    calls = {
+        "forward_dual_gemm": (lambda: _abi.check(L.fsw_swiglu_forward(p(xd), p(wgd), p(wud), p(out), p(g), p(u), T, D, I, D, I, I, 0, stream)), 4.0 * T * D * I),
+        "elementwise_backward": (lambda: _abi.check(L.fsw_elementwise_backward(p(dout), p(g), p(u), p(dU), p(dG), T * I, 0, stream)), None),
+        "input_grad_dual_gemm": (lambda: _abi.check(L.fsw_input_grad(p(dG), p(dU), p(wgd), p(wud), p(dx), T, D, I, I, I, D, 0, stream)), 4.0 * T * D * I),
+        "weight_grad_dual_gemm": (lambda: _abi.check(L.fsw_weight_grad(p(xd), p(dU), p(dG), p(dWu), p(dWg), T, D, I, D, I, I, 0, stream)), 4.0 * T * D * I),
+    }
+    kernels = {}
+    for name, (fn, flop) in calls.items():
+        ms = gpu_time_ms(fn, iters=max(5, args.steps))
+        rec = {"ms": round(ms, 4)}
+        if flop is not None:
+            rec["tflops"] = round(flop / ms / 1e9, 1)
+            rec["frac_mfma_peak"] = round(flop / ms / 1e9 / PEAK_BF16_TFLOPS, 4)
+        else:
+            rec["gbs"] = round(10.0 * T * I / ms / 1e6, 1)  # 3 reads + 2 writes of 2 bytes per element
+            rec["frac_hbm_peak"] = round(rec["gbs"] / PEAK_HBM_GBS, 4)
+        kernels[name] = rec
+    gemm_names = [k for k in kernels if "tflops" in kernels[k]]
+    dominant = max(gemm_names, key=lambda k: kernels[k]["ms"])
+    achieved = 4.0 * T * D * I / kernels[dominant]["ms"] / 1e9
+    roofline = {
+        "kernel": dominant,
+        "bound": "mfma",
+        "achieved": round(achieved, 1),
+        "peak": PEAK_BF16_TFLOPS,
+        "unit": "TFLOP/s",
+        "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
+        "traffic": None,
+    }
+
+    result = {
+        "metric": "fwd+bwd TFLOP/s & % bf16 MFMA peak, 8192 tok, d=4096->12288",
+        "value": round(tflops, 1),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "C2: bf16 FusedSwiGLU fwd+bwd, x [4,2048,4096], Wg/Wu [4096,12288], "
+                               "dout ~ N(0,1), fp32 MFMA accumulate", "tokens": T, "d_model": D,
+                   "d_intermediate": I, "flop_per_step": flop_step},
+        "pct_of_bf16_mfma_peak": round(100.0 * tflops / PEAK_BF16_TFLOPS, 2),
+        "roofline": roofline,
+        "kernels": kernels,
+    }
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, device=dev, dtype=torch.uint8).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
+    # ---- skinny-M forward (weight streaming, HBM bound), forward only, no pre-activation stores
+    if not args.no_extra:
+        del out, g, u, dG, dU, dx, dWg, dWu
+        D4, I4 = 8192, 28672
+        w_sets = [((torch.randn(D4, I4, device=dev, dtype=dt) / D4 ** 0.5), (torch.randn(D4, I4, device=dev, dtype=dt) / D4 ** 0.5))
+                  for _ in range(2)]
+        skinny = []
+        for M in (16, 64, 256):
+            xs = torch.randn(M, D4, device=dev, dtype=dt)
+            os_ = torch.empty(M, I4, device=dev, dtype=dt)
+            state = {"i": 0}
+
+            def fwd():
+                a, b = w_sets[state["i"] & 1]  # alternate weight sets: nothing stays cache resident
+                state["i"] += 1
+                _abi.check(L.fsw_swiglu_forward(p(xs), p(a), p(b), p(os_), None, None, M, D4, I4, D4, I4, I4, 0, stream))
+
+            ms = gpu_time_ms(fwd, iters=20)
+            nbytes = 2.0 * (2 * D4 * I4 + M * D4 + M * I4)
+            skinny.append({"M": M, "ms": round(ms, 4), "gbs": round(nbytes / ms / 1e6, 1),
+                           "frac_hbm_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4),
+                           "tflops": round(4.0 * M * D4 * I4 / ms / 1e9, 1)})
+        result["skinny_forward"] = {"workload": "C4: bf16 forward, x [M,8192], Wg/Wu [8192,28672]", "bound": "hbm",
+                                    "peak_gbs": PEAK_HBM_GBS, "runs": skinny}
+        del w_sets
+
+    # ---- CPU baseline: the eager fp32 SwiGLU of the reference's test on this machine's host cores
+    if not args.no_cpu_baseline:
+        from oracle import swiglu_oracle as osw
+
+        torch.manual_seed(0)
+        Bc, Sc, Dc, Ic = 4, 2048, 1024, 3072
+        xc = torch.randn(Bc, Sc, Dc)
+        wgc, wuc = torch.randn(Dc, Ic) / Dc ** 0.5, torch.randn(Dc, Ic) / Dc ** 0.5
+        dyc = torch.randn(Bc, Sc, Ic)
+        osw.eager_torch_fwd_bwd(xc, wgc, wuc, dyc)  # warm-up
+        best = float("inf")
+        t_all = time.perf_counter()
+        reps = 0
+        while reps < 3 or (time.perf_counter() - t_all < 10.0 and reps < 30):
+            t1 = time.perf_counter()
+            osw.eager_torch_fwd_bwd(xc, wgc, wuc, dyc)
+            best = min(best, time.perf_counter() - t1)
+            reps += 1
+        fl = 12.0 * Bc * Sc * Dc * Ic
+        result["cpu_baseline"] = {
+            "value": round(fl / best / 1e12, 4),
+            "unit": "TFLOP/s",
+            "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"C1: eager fp32 PyTorch SwiGLU fwd+bwd, x [4,2048,1024], W [1024,3072]; best of {reps} "
+                      f"after a warm-up, {best * 1e3:.1f} ms; os.cpu_count()={os.cpu_count()}",
+        }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

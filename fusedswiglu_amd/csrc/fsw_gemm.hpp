@@ -29,7 +29,10 @@ struct GemmParams {
 };
 
 constexpr int kThreads = 512;
-constexpr int kStages = 4;
+#ifndef FSW_STAGES
+#define FSW_STAGES 4
+#endif
+constexpr int kStages = FSW_STAGES;
 constexpr int kRegionBytes = 16384;           // one operand tile of one stage
 constexpr int kStageBytes = 2 * kRegionBytes;  // A region then B region
 constexpr int kTileM = 256;
@@ -100,8 +103,13 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
   for (int i = 0; i < 2; i++) {
     const int j = wave + 8 * i;
     if constexpr (A_KC) {
+#ifdef FSW_DBG_KC128
+      const int row = 8 * j + (lane >> 3);
+      const int c = (lane & 7);
+#else
       const int row = 16 * j + (lane >> 2);
       const int c = (lane & 3) ^ ((lane >> 4) & 3);
+#endif
       sa[i].lane_off = (unsigned)row * (unsigned)p.lda * 2u + c * 16u;
       sa[i].klim = (m0 + row < p.M) ? p.K - c * 8 : -0x40000000;
       a_base[i] = (const char*)p.a0 + (size_t)m0 * p.lda * 2;
@@ -117,8 +125,13 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
       a_base2[i] = a_base[i];
     }
     if constexpr (B_KC) {
+#ifdef FSW_DBG_KC128
+      const int row = 8 * j + (lane >> 3);
+      const int c = (lane & 7);
+#else
       const int row = 16 * j + (lane >> 2);
       const int c = (lane & 3) ^ ((lane >> 4) & 3);
+#endif
       sb[i].lane_off = (unsigned)row * (unsigned)p.ldb * 2u + c * 16u;
       sb[i].klim = (n0 + row < p.N) ? p.K - c * 8 : -0x40000000;
       b_base[i] = (const char*)p.b0 + (size_t)n0 * p.ldb * 2;
@@ -140,7 +153,7 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
     const int pass = (MODE == kDx && kt >= kt1) ? 1 : 0;
     const int ktl = kt - pass * kt1;
     const int k0 = ktl * kBK;
-    const unsigned stage_addr = smem_addr + (unsigned)(kt & (kStages - 1)) * kStageBytes;
+    const unsigned stage_addr = smem_addr + (unsigned)(kt % kStages) * kStageBytes;
 #pragma unroll
     for (int i = 0; i < 2; i++) {
       const int j = wave + 8 * i;
@@ -165,42 +178,68 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[a][q][r] = 0.f;
 
-  // ---- prologue: up to three stages in flight
+  // ---- main loop: two groups of four waves (one per SIMD each) run half a step out of phase.
+  // While one group reads its fragments of a stage from LDS (and issues its share of the loads
+  // for the stage three ahead), the other group issues the 16 MFMAs of the stage it read one
+  // phase earlier, so the matrix cores of every SIMD always have a wave to serve.  Phases are
+  // separated by workgroup barriers; group 1 enters one barrier late and leaves one early.
+  const int grp = wave >> 2;
+  auto phase_barrier = [&](int kt) {
+    // stage kt+1 must have landed (for every wave's share) before the next phase reads it;
+    // stages kt+2 and kt+3, if they exist, may stay in flight
+    const int ahead = min(kt_total - 2 - kt, kStages - 2);
+    if (ahead >= 3) wait_vmcnt_and_barrier<12>();
+    else if (ahead == 2) wait_vmcnt_and_barrier<8>();
+    else if (ahead == 1) wait_vmcnt_and_barrier<4>();
+    else wait_vmcnt_and_barrier<0>();
+  };
 #pragma unroll
   for (int s = 0; s < kStages - 1; s++)
     if (s < kt_total) issue(s);
+  phase_barrier(-1);
+  if (grp == 1) wait_vmcnt_and_barrier<63>();
 
   for (int kt = 0; kt < kt_total; kt++) {
-    const int ahead = kt_total - 1 - kt;  // stages issued beyond this one that may stay in flight
-    if (ahead >= 2) wait_vmcnt_and_barrier<8>();
-    else if (ahead == 1) wait_vmcnt_and_barrier<4>();
-    else wait_vmcnt_and_barrier<0>();
-    if (kt + kStages - 1 < kt_total) issue(kt + kStages - 1);
-
-    const FSW_LDS char* ra = smem_l + (kt & (kStages - 1)) * kStageBytes;
+    const FSW_LDS char* ra = smem_l + (kt % kStages) * kStageBytes;
     const FSW_LDS char* rb = ra + kRegionBytes;
+    i16x8 fq[2][4], fp[2][2];
+#ifdef FSW_DBG_NO_LDSREAD
+    for (int ks = 0; ks < 2; ks++) { for (int q = 0; q < 4; q++) fq[ks][q] = (i16x8)(short)(kt + q); for (int a = 0; a < 2; a++) fp[ks][a] = (i16x8)(short)(kt + a); }
+    if (p.M < 0)
+#endif
 #pragma unroll
     for (int ks = 0; ks < 2; ks++) {
-      i16x8 fq[4], fp[2];
 #pragma unroll
       for (int q = 0; q < 4; q++) {
-        if constexpr (A_KC) fq[q] = read_frag_kc(ra, wm * 128 + q * 32, ks, lane);
-        else fq[q] = read_frag_mc(ra + wm * kMcPanelBytes, q, ks, lane);
+        if constexpr (A_KC) fq[ks][q] = read_frag_kc(ra, wm * 128 + q * 32, ks, lane);
+        else fq[ks][q] = read_frag_mc(ra + wm * kMcPanelBytes, q, ks, lane);
       }
 #pragma unroll
       for (int a = 0; a < 2; a++) {
-        if constexpr (B_KC) fp[a] = read_frag_kc(rb, wn * 64 + a * 32, ks, lane);
-        else fp[a] = read_frag_mc(rb + a * kMcPanelBytes, wn, ks, lane);
+        if constexpr (B_KC) fp[ks][a] = read_frag_kc(rb, wn * 64 + a * 32, ks, lane);
+        else fp[ks][a] = read_frag_mc(rb + a * kMcPanelBytes, wn, ks, lane);
       }
+    }
+#ifndef FSW_DBG_NO_DMA
+    if (kt + kStages - 1 < kt_total) issue(kt + kStages - 1);
+#endif
+    phase_barrier(kt);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++)
 #pragma unroll
       for (int q = 0; q < 4; q++)
 #pragma unroll
-        for (int a = 0; a < 2; a++) acc[a][q] = E::mfma(fp[a], fq[q], acc[a][q]);
-    }
+        for (int a = 0; a < 2; a++) acc[a][q] = E::mfma(fp[ks][a], fq[ks][q], acc[a][q]);
+    __builtin_amdgcn_sched_barrier(0);
+    if (!(grp == 1 && kt == kt_total - 1)) phase_barrier(kt);
   }
 
   // ---- epilogue.  acc[a][q][r] of lane l is row  m0 + wm*128 + q*32 + (l & 31)  and column
   //      cbase(a) + 8*(r >> 2) + 4*(l >> 5) + (r & 3): four consecutive columns per 8-byte store.
+#ifdef FSW_DBG_NO_STORE
+  if (p.M > 0 && acc[0][0][0] != 123.456f) return;
+#endif
   const int mrow = m0 + wm * 128 + (lane & 31);
   const int ncol_l = 4 * (lane >> 5);
 #pragma unroll
