@@ -26,8 +26,13 @@ typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 struct BF16 {
   using vec8 = bf16x8;
   static FSW_DEV f32x16 mfma(i16x8 a, i16x8 b, f32x16 c) {
+#ifdef FSW_AGPR_ACC
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    return c;
+#else
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
                                                    __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+#endif
   }
   static FSW_DEV float to_float(unsigned short v) { return __uint_as_float((unsigned)v << 16); }
   // round-to-nearest-even; NaN stays NaN
@@ -91,7 +96,13 @@ FSW_DEV void load16_to_lds(i32x4 rsrc, unsigned voffset, unsigned lds_addr) {
 template <int N>
 FSW_DEV void wait_vmcnt_and_barrier() {
   static_assert(N >= 0 && N < 64, "vmcnt is 6 bits");
+#ifdef FSW_BARRIER_LGKM
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "n"(N) : "memory");
+#else
+  // LDS reads issued before the barrier may still be in flight: their consumers carry their own
+  // lgkmcnt waits, and no LDS slot is overwritten until a full step after it was last read
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" : : "n"(N) : "memory");
+#endif
 }
 
 // ---- LDS tile formats -------------------------------------------------------

@@ -6,8 +6,12 @@
 //
 // One workgroup = 8 wavefronts (2 along M x 4 along N) = one 256 x 256 fp32 accumulator tile
 // (kFwd / kDw: 256 rows x 128 columns of EACH of the two results, sharing the A tile).
-// The reduction advances 32 elements per step through a 4-deep ring of 32 KiB LDS stages that
-// is filled by direct global->LDS loads three steps ahead of the MFMAs.
+// The reduction advances 32 elements per step.  Operand tiles are brought in by direct
+// global->LDS loads several steps ahead of the MFMAs and kept in LDS rings:
+//   * an m/n-contiguous ("MC") operand uses a ring of four 16 KiB slots, one per step;
+//   * a k-contiguous ("KC") operand is fetched 64 k-elements (one full 128-byte line per row) at a
+//     time into a ring of 32 KiB areas, each serving two consecutive steps.  Fetching half lines
+//     (64 bytes per row per step) halves the throughput of the texture-address path.
 #pragma once
 #include "fsw_common.hpp"
 
@@ -29,30 +33,46 @@ struct GemmParams {
 };
 
 constexpr int kThreads = 512;
-#ifndef FSW_STAGES
-#define FSW_STAGES 4
-#endif
-constexpr int kStages = FSW_STAGES;
-constexpr int kRegionBytes = 16384;           // one operand tile of one stage
-constexpr int kStageBytes = 2 * kRegionBytes;  // A region then B region
 constexpr int kTileM = 256;
+constexpr int kMcSlots = 4;
+constexpr int kMcSlotBytes = 2 * kMcPanelBytes;  // two 128-column panels: 16 KiB
+constexpr int kKcAreaBytes = 256 * 128;          // 256 rows x 64 k-elements: 32 KiB
+
+#ifndef FSW_KC_AREAS_A
+#define FSW_KC_AREAS_A 3
+#endif
+
 template <int MODE>
-constexpr int tile_n() {
-  return MODE == kDx ? 256 : 128;
-}
+struct Cfg {
+  static constexpr bool kAKc = (MODE != kDw);
+  static constexpr bool kBKc = (MODE == kDx);
+  static constexpr int kTileN = (MODE == kDx) ? 256 : 128;
+  // KC rings: number of 32 KiB areas.  160 KiB of LDS in all for kFwd and kDx, 128 KiB for kDw.
+  static constexpr int kAreasA = FSW_KC_AREAS_A;
+  static constexpr int kAreasB = 2;
+  static constexpr int kBytesA = kAKc ? kAreasA * kKcAreaBytes : kMcSlots * kMcSlotBytes;
+  static constexpr int kBytesB = kBKc ? kAreasB * kKcAreaBytes : kMcSlots * kMcSlotBytes;
+  // how many steps ahead of its use an operand's loads are issued
+  static constexpr int kAheadA = kAKc ? 2 * (kAreasA - 1) : kMcSlots - 1;
+  static constexpr int kAheadB = kBKc ? 2 * (kAreasB - 1) : kMcSlots - 1;
+  static constexpr int kAheadMax = kAheadA > kAheadB ? kAheadA : kAheadB;
+};
 
 // ---- fragment reads -----------------------------------------------------------
-// K-contiguous tile: lane l gets row (l & 31), k = ks*16 + 8*(l >> 5) .. +8 in one ds_read_b128.
-FSW_DEV i16x8 read_frag_kc(const FSW_LDS char* region, int row_base, int ks, int lane) {
+// KC area: 256 rows x 128 bytes; the 16-byte chunk c of row r sits at chunk position
+// c ^ ((r >> 1) & 7), so that 16 consecutive rows cover all 64 banks for a fixed c.
+// Lane l gets row (l & 31), k = half*32 + ks*16 + 8*(l >> 5) .. +8 in one ds_read_b128.
+FSW_DEV i16x8 read_frag_kc(const FSW_LDS char* area, int row_base, int half, int ks, int lane) {
   const int row = row_base + (lane & 31);
-  const int chunk = (ks * 2 + (lane >> 5)) ^ ((lane >> 2) & 3);
-  return *(const FSW_LDS i16x8*)(region + row * kKcRowBytes + chunk * 16);
+  const int chunk = (half * 4 + ks * 2 + (lane >> 5)) ^ ((lane >> 1) & 7);
+  return *(const FSW_LDS i16x8*)(area + row * 128 + chunk * 16);
 }
 
-// M/N-contiguous panel: two transposing reads.  Within each group of 16 lanes, lane j supplies the
-// address of 4 consecutive columns (j & 3)*4.. of k-row (j >> 2); the hardware hands lane i the
-// column i of those four k-rows.  Lane groups 0/1 cover columns 0-15 / 16-31 of the 32-column
-// fragment, groups 2/3 the same columns 8 k-rows further on -- the MFMA operand layout.
+// MC panel: 32 k-rows x 256 bytes; the 64-byte block b of k-row k sits at block position b ^ (k & 3).
+// Two transposing reads.  Within each group of 16 lanes, lane j supplies the address of 4
+// consecutive columns (j & 3)*4.. of k-row (j >> 2); the hardware hands lane i the column i of
+// those four k-rows.  Lane groups 0/1 cover columns 0-15 / 16-31 of the 32-column fragment,
+// groups 2/3 the same columns 8 k-rows further on -- the MFMA operand layout.
 FSW_DEV i16x8 read_frag_mc(const FSW_LDS char* panel, int block64, int ks, int lane) {
   const int grp = lane >> 4, j = lane & 15;
   const int krow = ks * 16 + 8 * (grp >> 1) + (j >> 2);
@@ -65,18 +85,56 @@ FSW_DEV i16x8 read_frag_mc(const FSW_LDS char* panel, int block64, int ks, int l
   return r;
 }
 
-// ---- per-thread description of one direct-to-LDS load -----------------------------
-struct DmaSlot {
-  unsigned lane_off;  // byte offset of this lane's 16 bytes relative to the moving base
-  int klim;           // the load is in range while k0 < klim
+// ---- per-wave description of an operand's direct-to-LDS loads -----------------------
+// KC operand: a wave issues 4 instructions per area (rows 8*(wave + 8i) .. +8, 128 bytes each).
+struct KcLoader {
+  unsigned lane_off;   // byte offset of this lane's 16 bytes for i = 0, relative to the moving base
+  unsigned row_step;   // bytes between the rows of consecutive i (64 rows)
+  int klim[4];         // instruction i is in range while k0 < klim[i]
+  const char* base0;   // tile origin at k = 0 (first pass)
+  const char* base1;   // second pass (kDx), else the same
 };
+// MC operand: 2 instructions per slot (wave, wave + 8): 4 k-rows x 256 bytes of panel (j >> 3).
+struct McLoader {
+  unsigned lane_off[2];
+  int klim[2];
+  const char* base[2];
+  size_t kstep;  // bytes per 32 k-rows
+};
+
+FSW_DEV void kc_setup(KcLoader& L, const void* p0, const void* p1, int row0, int rows_total, int K,
+                      int ld, int wave, int lane) {
+  const int row = 8 * wave + (lane >> 3);
+  const int c = (lane & 7) ^ ((((wave & 1) << 2) + (lane >> 4)) & 7);
+  L.lane_off = (unsigned)row * (unsigned)ld * 2u + c * 16u;
+  L.row_step = 64u * (unsigned)ld * 2u;
+#pragma unroll
+  for (int i = 0; i < 4; i++) L.klim[i] = (row0 + row + 64 * i < rows_total) ? K - c * 8 : -0x40000000;
+  L.base0 = (const char*)p0 + (size_t)row0 * ld * 2;
+  L.base1 = (const char*)p1 + (size_t)row0 * ld * 2;
+}
+
+FSW_DEV void mc_setup(McLoader& L, const void* p_panel0, const void* p_panel1, int col0_panel0,
+                      int col0_panel1, int cols_total, int K, int ld, int wave, int lane) {
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const int j = wave + 8 * i;
+    const int row = 4 * (j & 7) + (lane >> 4);
+    const int col = (((lane >> 2) & 3) ^ ((lane >> 4) & 3)) * 32 + (lane & 3) * 8;
+    const int col0 = (j >> 3) ? col0_panel1 : col0_panel0;
+    L.lane_off[i] = (unsigned)row * (unsigned)ld * 2u + col * 2u;
+    L.klim[i] = (col0 + col < cols_total) ? K - row : -0x40000000;
+    L.base[i] = (const char*)((j >> 3) ? p_panel1 : p_panel0) + (size_t)col0 * 2;
+  }
+  L.kstep = (size_t)kBK * ld * 2;
+}
 
 template <typename E, int MODE>
 __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
-  __shared__ __attribute__((aligned(1024))) char smem[kStages * kStageBytes];
-  constexpr bool A_KC = (MODE != kDw);
-  constexpr bool B_KC = (MODE == kDx);
-  constexpr int TN = tile_n<MODE>();
+  using C = Cfg<MODE>;
+  __shared__ __attribute__((aligned(1024))) char smem[C::kBytesA + C::kBytesB];
+  constexpr bool A_KC = C::kAKc, B_KC = C::kBKc;
+  constexpr int TN = C::kTileN;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -84,89 +142,88 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
   const int wm = wave >> 2, wn = wave & 3;
 
   const TileCoord tc = xcd_tile_order(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m);
+#ifdef FSW_DBG_SAMETILE
+  const int m0 = (tc.tm & (FSW_DBG_SAMETILE - 1)) * kTileM;
+  const int n0 = (tc.tn & (FSW_DBG_SAMETILE - 1)) * TN;
+#else
   const int m0 = tc.tm * kTileM;
   const int n0 = tc.tn * TN;
+#endif
 
-  const int kt1 = (p.K + kBK - 1) / kBK;
+  // steps per pass; kDx makes two passes (dG.Wg^T then dU.Wu^T) and keeps pairs of steps inside a pass
+  const int kt1 = (MODE == kDx) ? (((p.K + kBK - 1) / kBK + 1) & ~1) : (p.K + kBK - 1) / kBK;
   const int kt_total = (MODE == kDx) ? 2 * kt1 : kt1;
 
-  const unsigned smem_addr = (unsigned)(uintptr_t)(FSW_LDS char*)smem;
-  const FSW_LDS char* smem_l = (const FSW_LDS char*)smem;
+  const unsigned smem_a = (unsigned)(uintptr_t)(FSW_LDS char*)smem;
+  const unsigned smem_b = smem_a + C::kBytesA;
+  const FSW_LDS char* lds_a = (const FSW_LDS char*)smem;
+  const FSW_LDS char* lds_b = lds_a + C::kBytesA;
 
-  // ---- DMA set-up: every wave issues instructions {wave, wave + 8} of each 16-instruction region
-  DmaSlot sa[2], sb[2];
-  const char* a_base[2];  // per instruction: pointer of the tile origin at k0 = 0 (uniform)
-  const char* b_base[2];
-  const char* a_base2[2];  // kDx second pass
-  const char* b_base2[2];
+  KcLoader ka, kb;
+  McLoader ma, mb;
+  if constexpr (A_KC) kc_setup(ka, p.a0, MODE == kDx ? p.a1 : p.a0, m0, p.M, p.K, p.lda, wave, lane);
+  else mc_setup(ma, p.a0, p.a0, m0, m0 + 128, p.M, p.K, p.lda, wave, lane);
+  if constexpr (B_KC) kc_setup(kb, p.b0, p.b1, n0, p.N, p.K, p.ldb, wave, lane);
+  else mc_setup(mb, p.b0, p.b1, n0, n0, p.N, p.K, p.ldb, wave, lane);
+
+  // loads of the pair of steps (pr, pr+1) of a KC operand into area (pr/2) % areas
+  auto issue_kc = [&](const KcLoader& L, int pr, int areas, unsigned lds_base) {
+    if (pr < 0 || pr >= kt_total) return;
+    const int pass = (MODE == kDx && pr >= kt1) ? 1 : 0;
+    const int k0 = (pr - pass * kt1) * kBK;
+    const i32x4 rs = make_rsrc((pass ? L.base1 : L.base0) + (size_t)k0 * 2);
+    const unsigned dst = lds_base + (unsigned)((pr >> 1) % areas) * kKcAreaBytes + wave * 1024;
 #pragma unroll
-  for (int i = 0; i < 2; i++) {
-    const int j = wave + 8 * i;
-    if constexpr (A_KC) {
-#ifdef FSW_DBG_KC128
-      const int row = 8 * j + (lane >> 3);
-      const int c = (lane & 7);
-#else
-      const int row = 16 * j + (lane >> 2);
-      const int c = (lane & 3) ^ ((lane >> 4) & 3);
-#endif
-      sa[i].lane_off = (unsigned)row * (unsigned)p.lda * 2u + c * 16u;
-      sa[i].klim = (m0 + row < p.M) ? p.K - c * 8 : -0x40000000;
-      a_base[i] = (const char*)p.a0 + (size_t)m0 * p.lda * 2;
-      a_base2[i] = (const char*)p.a1 + (size_t)m0 * p.lda * 2;
-    } else {
-      // kDw: panel (j >> 3) holds x columns m0 + 128*(j >> 3) ..
-      const int row = 4 * (j & 7) + (lane >> 4);
-      const int col = (((lane >> 2) & 3) ^ ((lane >> 4) & 3)) * 32 + (lane & 3) * 8;
-      const int col0 = m0 + 128 * (j >> 3);
-      sa[i].lane_off = (unsigned)row * (unsigned)p.lda * 2u + col * 2u;
-      sa[i].klim = (col0 + col < p.M) ? p.K - row : -0x40000000;
-      a_base[i] = (const char*)p.a0 + (size_t)col0 * 2;
-      a_base2[i] = a_base[i];
+    for (int i = 0; i < 4; i++) {
+      const unsigned off = (k0 < L.klim[i]) ? L.lane_off + i * L.row_step : kOobOffset;
+      load16_to_lds(rs, off, dst + i * 8192);
     }
-    if constexpr (B_KC) {
-#ifdef FSW_DBG_KC128
-      const int row = 8 * j + (lane >> 3);
-      const int c = (lane & 7);
-#else
-      const int row = 16 * j + (lane >> 2);
-      const int c = (lane & 3) ^ ((lane >> 4) & 3);
-#endif
-      sb[i].lane_off = (unsigned)row * (unsigned)p.ldb * 2u + c * 16u;
-      sb[i].klim = (n0 + row < p.N) ? p.K - c * 8 : -0x40000000;
-      b_base[i] = (const char*)p.b0 + (size_t)n0 * p.ldb * 2;
-      b_base2[i] = (const char*)p.b1 + (size_t)n0 * p.ldb * 2;
-    } else {
-      // panel 0 = first B matrix, panel 1 = second, same 128 columns n0..
-      const int row = 4 * (j & 7) + (lane >> 4);
-      const int col = (((lane >> 2) & 3) ^ ((lane >> 4) & 3)) * 32 + (lane & 3) * 8;
-      sb[i].lane_off = (unsigned)row * (unsigned)p.ldb * 2u + col * 2u;
-      sb[i].klim = (n0 + col < p.N) ? p.K - row : -0x40000000;
-      b_base[i] = (const char*)((j >> 3) ? p.b1 : p.b0) + (size_t)n0 * 2;
-      b_base2[i] = b_base[i];
-    }
-  }
-  const size_t a_kstep = A_KC ? (size_t)kBK * 2 : (size_t)kBK * p.lda * 2;
-  const size_t b_kstep = B_KC ? (size_t)kBK * 2 : (size_t)kBK * p.ldb * 2;
-
-  auto issue = [&](int kt) {
-    const int pass = (MODE == kDx && kt >= kt1) ? 1 : 0;
-    const int ktl = kt - pass * kt1;
-    const int k0 = ktl * kBK;
-    const unsigned stage_addr = smem_addr + (unsigned)(kt % kStages) * kStageBytes;
+  };
+  // loads of step s of an MC operand into slot s % 4
+  auto issue_mc = [&](const McLoader& L, int s, unsigned lds_base) {
+    if (s < 0 || s >= kt_total) return;
+    const int k0 = s * kBK;
+    const unsigned dst = lds_base + (unsigned)(s & (kMcSlots - 1)) * kMcSlotBytes + wave * 1024;
 #pragma unroll
     for (int i = 0; i < 2; i++) {
-      const int j = wave + 8 * i;
-      const char* ab = (pass ? a_base2[i] : a_base[i]) + (size_t)ktl * a_kstep;
-      const unsigned off = (k0 < sa[i].klim) ? sa[i].lane_off : kOobOffset;
-      load16_to_lds(make_rsrc(ab), off, stage_addr + j * 1024);
+      const unsigned off = (k0 < L.klim[i]) ? L.lane_off[i] : kOobOffset;
+      load16_to_lds(make_rsrc(L.base[i] + (size_t)s * L.kstep), off, dst + i * 8192);
     }
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-      const int j = wave + 8 * i;
-      const char* bb = (pass ? b_base2[i] : b_base[i]) + (size_t)ktl * b_kstep;
-      const unsigned off = (k0 < sb[i].klim) ? sb[i].lane_off : kOobOffset;
-      load16_to_lds(make_rsrc(bb), off, stage_addr + kRegionBytes + j * 1024);
+  };
+  // everything a wave issues during step i (i < 0: prologue).  The order fixes the vmcnt arithmetic below.
+  auto issue_step = [&](int i) {
+    if ((i & 1) == 0) {
+      if constexpr (B_KC) issue_kc(kb, i + C::kAheadB, C::kAreasB, smem_b);
+      if constexpr (A_KC) issue_kc(ka, i + C::kAheadA, C::kAreasA, smem_a);
+    }
+    if constexpr (!A_KC) issue_mc(ma, i + C::kAheadA, smem_a);
+    if constexpr (!B_KC) issue_mc(mb, i + C::kAheadB, smem_b);
+  };
+  // Wait until this wave's share of step kt+1 has landed, then meet the other waves.  Loads complete in
+  // issue order, so it is enough to bound how many of the younger ones may still be in flight.  With
+  // three KC areas for A:
+  //   kFwd  after the MC slot of step kt+1 (issued during step kt-2) come one KC batch (4) and two MC
+  //         batches (2+2)                                                                    -> 8
+  //   kDw   two steps of 2+2                                                                 -> 8
+  //   kDx   step kt odd: after the B pair of kt+1 (issued first during step kt-1) comes only the A pair
+  //         issued with it -> 4;  kt even: nothing new is needed, this step's 8 loads are younger -> 12
+  // With two KC areas for A the A pair of step kt+1 is issued during step kt-1 as well:
+  //   kFwd  kt odd: after that A pair come MC(kt+2), MC(kt+3) -> 4;  kt even: as above -> 8
+  //   kDx   kt odd: the A pair is the youngest load -> 0;  kt even: this step's 8 loads -> 8
+  // Near the end of the reduction, where some of those loads no longer exist, wait for everything.
+  auto wait_next_step_and_barrier = [&](int kt) {
+#ifdef FSW_DBG_NOWAIT
+    if (kt < kt_total - 1) { wait_vmcnt_and_barrier<63>(); return; }
+#endif
+    if (kt + C::kAheadMax >= kt_total) { wait_vmcnt_and_barrier<0>(); return; }
+    if constexpr (MODE == kDx) {
+      if (kt & 1) wait_vmcnt_and_barrier<(C::kAreasA == 3 ? 4 : 0)>();
+      else wait_vmcnt_and_barrier<(C::kAreasA == 3 ? 12 : 8)>();
+    } else if constexpr (MODE == kFwd && C::kAreasA == 2) {
+      if (kt & 1) wait_vmcnt_and_barrier<4>();
+      else wait_vmcnt_and_barrier<8>();
+    } else {
+      wait_vmcnt_and_barrier<8>();
     }
   };
 
@@ -179,29 +236,37 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
       for (int r = 0; r < 16; r++) acc[a][q][r] = 0.f;
 
   // ---- main loop: two groups of four waves (one per SIMD each) run half a step out of phase.
-  // While one group reads its fragments of a stage from LDS (and issues its share of the loads
-  // for the stage three ahead), the other group issues the 16 MFMAs of the stage it read one
-  // phase earlier, so the matrix cores of every SIMD always have a wave to serve.  Phases are
-  // separated by workgroup barriers; group 1 enters one barrier late and leaves one early.
+  // While one group reads its fragments of a step from LDS (and issues its share of the loads for
+  // later steps), the other group issues the 16 MFMAs of the step it read one phase earlier, so the
+  // matrix cores of every SIMD always have a wave to serve.  Phases are separated by workgroup
+  // barriers; group 1 enters one barrier late and leaves one early.
   const int grp = wave >> 2;
-  auto phase_barrier = [&](int kt) {
-    // stage kt+1 must have landed (for every wave's share) before the next phase reads it;
-    // stages kt+2 and kt+3, if they exist, may stay in flight
-    const int ahead = min(kt_total - 2 - kt, kStages - 2);
-    if (ahead >= 3) wait_vmcnt_and_barrier<12>();
-    else if (ahead == 2) wait_vmcnt_and_barrier<8>();
-    else if (ahead == 1) wait_vmcnt_and_barrier<4>();
-    else wait_vmcnt_and_barrier<0>();
-  };
 #pragma unroll
-  for (int s = 0; s < kStages - 1; s++)
-    if (s < kt_total) issue(s);
-  phase_barrier(-1);
+  for (int i = -C::kAheadMax; i < 0; i++) issue_step(i);
+  wait_next_step_and_barrier(-1);
   if (grp == 1) wait_vmcnt_and_barrier<63>();
 
+#if FSW_DBG_TIMING == 4
+  const unsigned long long t_loop0 = __builtin_readcyclecounter();
+#endif
+#ifdef FSW_DBG_TIMING
+  unsigned long long* dbg = (unsigned long long*)p.c2;  // kDx/kDw leave c2 unused: harness passes a buffer
+  const bool dbg_on = (blockIdx.x == 8) && (lane == 0);
+#define FSW_STAMP(slot) do { if (kt >= 40 && kt < 48) { unsigned long long t_ = __builtin_readcyclecounter(); if (dbg_on) dbg[(wave * 8 + (kt - 40)) * 4 + (slot)] = t_; } } while (0)
+#else
+#define FSW_STAMP(slot) do {} while (0)
+#endif
   for (int kt = 0; kt < kt_total; kt++) {
-    const FSW_LDS char* ra = smem_l + (kt % kStages) * kStageBytes;
-    const FSW_LDS char* rb = ra + kRegionBytes;
+    const FSW_LDS char* ra;
+    const FSW_LDS char* rb;
+    if constexpr (A_KC) ra = lds_a + ((kt >> 1) % C::kAreasA) * kKcAreaBytes;
+    else ra = lds_a + (kt & (kMcSlots - 1)) * kMcSlotBytes;
+    if constexpr (B_KC) rb = lds_b + ((kt >> 1) % C::kAreasB) * kKcAreaBytes;
+    else rb = lds_b + (kt & (kMcSlots - 1)) * kMcSlotBytes;
+    const int half = kt & 1;
+#if FSW_DBG_TIMING == 1
+    FSW_STAMP(0);
+#endif
     i16x8 fq[2][4], fp[2][2];
 #ifdef FSW_DBG_NO_LDSREAD
     for (int ks = 0; ks < 2; ks++) { for (int q = 0; q < 4; q++) fq[ks][q] = (i16x8)(short)(kt + q); for (int a = 0; a < 2; a++) fp[ks][a] = (i16x8)(short)(kt + a); }
@@ -210,31 +275,75 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
 #pragma unroll
     for (int ks = 0; ks < 2; ks++) {
 #pragma unroll
+#ifdef FSW_DBG_HALFREADS
+      for (int q = 0; q < 2; q++) {
+#else
       for (int q = 0; q < 4; q++) {
-        if constexpr (A_KC) fq[ks][q] = read_frag_kc(ra, wm * 128 + q * 32, ks, lane);
+#endif
+        if constexpr (A_KC) fq[ks][q] = read_frag_kc(ra, wm * 128 + q * 32, half, ks, lane);
         else fq[ks][q] = read_frag_mc(ra + wm * kMcPanelBytes, q, ks, lane);
       }
 #pragma unroll
+#ifdef FSW_DBG_HALFREADS
+      for (int a = 0; a < 1; a++) {
+#else
       for (int a = 0; a < 2; a++) {
-        if constexpr (B_KC) fp[ks][a] = read_frag_kc(rb, wn * 64 + a * 32, ks, lane);
+#endif
+        if constexpr (B_KC) fp[ks][a] = read_frag_kc(rb, wn * 64 + a * 32, half, ks, lane);
         else fp[ks][a] = read_frag_mc(rb + a * kMcPanelBytes, wn, ks, lane);
       }
     }
-#ifndef FSW_DBG_NO_DMA
-    if (kt + kStages - 1 < kt_total) issue(kt + kStages - 1);
+#ifdef FSW_DBG_HALFREADS
+    // read only half of the A fragments and one B fragment; the rest are copies (timing experiment)
+    for (int ks = 0; ks < 2; ks++) { fq[ks][2] = fq[ks][0]; fq[ks][3] = fq[ks][1]; fp[ks][1] = fp[ks][0]; }
 #endif
-    phase_barrier(kt);
+#ifndef FSW_DBG_NO_DMA
+    issue_step(kt);
+#endif
+#if FSW_DBG_TIMING == 2
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    FSW_STAMP(1);
+#endif
+    wait_next_step_and_barrier(kt);
+#if FSW_DBG_TIMING == 1 || FSW_DBG_TIMING == 3
+    FSW_STAMP(2);
+#endif
     __builtin_amdgcn_sched_barrier(0);
+#ifdef FSW_SETPRIO
+    __builtin_amdgcn_s_setprio(FSW_SETPRIO);
+#endif
 #pragma unroll
     for (int ks = 0; ks < 2; ks++)
+#ifdef FSW_MFMA_ORDER_AQ
+#pragma unroll
+      for (int a = 0; a < 2; a++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+#else
 #pragma unroll
       for (int q = 0; q < 4; q++)
 #pragma unroll
-        for (int a = 0; a < 2; a++) acc[a][q] = E::mfma(fp[ks][a], fq[ks][q], acc[a][q]);
+        for (int a = 0; a < 2; a++) {
+#endif
+#ifdef FSW_DBG_NO_MFMA
+          { i16x8 t_ = fp[ks][a] ^ fq[ks][q]; i32x4 u_ = __builtin_bit_cast(i32x4, t_); acc[a][q][0] += __int_as_float(u_.x ^ u_.y ^ u_.z ^ u_.w); }
+#else
+          acc[a][q] = E::mfma(fp[ks][a], fq[ks][q], acc[a][q]);
+#endif
+        }
+#ifdef FSW_SETPRIO
+    __builtin_amdgcn_s_setprio(0);
+#endif
     __builtin_amdgcn_sched_barrier(0);
-    if (!(grp == 1 && kt == kt_total - 1)) phase_barrier(kt);
+#if FSW_DBG_TIMING == 2 || FSW_DBG_TIMING == 3
+    FSW_STAMP(3);
+#endif
+    if (!(grp == 1 && kt == kt_total - 1)) wait_vmcnt_and_barrier<63>();
   }
 
+#if FSW_DBG_TIMING == 4
+  { const unsigned long long t_loop1 = __builtin_readcyclecounter(); if (lane == 0 && (blockIdx.x & 255) == 8) { dbg[wave * 2] = t_loop1 - t_loop0; dbg[wave * 2 + 1] = kt_total; } }
+#endif
   // ---- epilogue.  acc[a][q][r] of lane l is row  m0 + wm*128 + q*32 + (l & 31)  and column
   //      cbase(a) + 8*(r >> 2) + 4*(l >> 5) + (r & 3): four consecutive columns per 8-byte store.
 #ifdef FSW_DBG_NO_STORE

@@ -29,7 +29,7 @@ bool fast_path_ok_weight_grad(const Problem& p) {
 
 template <int MODE>
 static hipError_t launch(int dtype, GemmParams g, hipStream_t s) {
-  constexpr int TN = tile_n<MODE>();
+  constexpr int TN = Cfg<MODE>::kTileN;
   g.tiles_m = (g.M + kTileM - 1) / kTileM;
   g.tiles_n = (g.N + TN - 1) / TN;
   g.group_m = 8;
