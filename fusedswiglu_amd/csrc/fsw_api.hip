@@ -101,6 +101,7 @@ int fsw_swiglu_forward(const void* x, const void* w_gate, const void* w_up, void
   p.x = x; p.wg = w_gate; p.wu = w_up; p.out = out; p.g = xw_gate; p.u = xw_up;
   p.T = T; p.D = D; p.I = I; p.ldx = ldx; p.ldw = ldw; p.ldo = ldo;
   hipStream_t s = (hipStream_t)stream;
+  if (!g_force_edge.load() && fsw::skinny_forward_ok(p)) return launched(fn, fsw::launch_forward_skinny(dtype, p, s));
   if (!g_force_edge.load() && fsw::fast_path_ok_forward(p)) return launched(fn, fsw::launch_forward_fast(dtype, p, s));
   return launched(fn, fsw::launch_forward_generic(dtype, p, s));
 }

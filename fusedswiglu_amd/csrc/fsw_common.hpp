@@ -83,11 +83,14 @@ FSW_DEV i32x4 make_rsrc(const void* base, unsigned num_records = 0x7fffffffu) {
 // (the LDS destination of a wave is contiguous by lane; lds_addr is wave-uniform).
 // Counted by vmcnt like any vector load; the compiler does not track it, so every consumer
 // must be fenced with wait_vmcnt<N>() + a workgroup barrier.
+#ifndef FSW_LOAD_MOD
+#define FSW_LOAD_MOD ""
+#endif
 FSW_DEV void load16_to_lds(i32x4 rsrc, unsigned voffset, unsigned lds_addr) {
   asm volatile(
       "s_mov_b32 m0, %0\n\t"
       "s_nop 0\n\t"
-      "buffer_load_dwordx4 %1, %2, 0 offen lds"
+      "buffer_load_dwordx4 %1, %2, 0 offen " FSW_LOAD_MOD "lds"
       :
       : "s"(lds_addr), "v"(voffset), "s"(rsrc)
       : "memory");

@@ -4,7 +4,7 @@
 //   kDx   dx  = dG Wg^T + dU Wu^T        A = dG | dU [T,I] (k-contiguous), B = Wg | Wu [D,I] rows (k-contiguous)
 //   kDw   dWg = x^T dG, dWu = x^T dU     A = x [T,D] (m-contiguous), B = dG | dU [T,I] (n-contiguous)
 //
-// One workgroup = 8 wavefronts (2 along M x 4 along N) = one 256 x 256 fp32 accumulator tile
+// One workgroup = 8 wavefronts (4 along M x 2 along N) = one 256 x 256 fp32 accumulator tile
 // (kFwd / kDw: 256 rows x 128 columns of EACH of the two results, sharing the A tile).
 // The reduction advances 32 elements per step.  Operand tiles are brought in by direct
 // global->LDS loads several steps ahead of the MFMAs and kept in LDS rings:
@@ -139,16 +139,11 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave >> 2, wn = wave & 3;
+  const int wm = wave >> 1, wn = wave & 1;  // 4 waves along M x 2 along N
 
   const TileCoord tc = xcd_tile_order(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m);
-#ifdef FSW_DBG_SAMETILE
-  const int m0 = (tc.tm & (FSW_DBG_SAMETILE - 1)) * kTileM;
-  const int n0 = (tc.tn & (FSW_DBG_SAMETILE - 1)) * TN;
-#else
   const int m0 = tc.tm * kTileM;
   const int n0 = tc.tn * TN;
-#endif
 
   // steps per pass; kDx makes two passes (dG.Wg^T then dU.Wu^T) and keeps pairs of steps inside a pass
   const int kt1 = (MODE == kDx) ? (((p.K + kBK - 1) / kBK + 1) & ~1) : (p.K + kBK - 1) / kBK;
@@ -212,9 +207,6 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
   //   kDx   kt odd: the A pair is the youngest load -> 0;  kt even: this step's 8 loads -> 8
   // Near the end of the reduction, where some of those loads no longer exist, wait for everything.
   auto wait_next_step_and_barrier = [&](int kt) {
-#ifdef FSW_DBG_NOWAIT
-    if (kt < kt_total - 1) { wait_vmcnt_and_barrier<63>(); return; }
-#endif
     if (kt + C::kAheadMax >= kt_total) { wait_vmcnt_and_barrier<0>(); return; }
     if constexpr (MODE == kDx) {
       if (kt & 1) wait_vmcnt_and_barrier<(C::kAreasA == 3 ? 4 : 0)>();
@@ -227,35 +219,28 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
     }
   };
 
-  f32x16 acc[2][4];
+  // acc[pp][q]: 32x32 block of rows wm*64 + q*32.. and column block pp of this wave:
+  //   kFwd/kDw  pp = 2*a + p: matrix a (gate | up), columns wn*64 + p*32..
+  //   kDx       columns wn*128 + pp*32..
+  f32x16 acc[4][2];
 #pragma unroll
-  for (int a = 0; a < 2; a++)
+  for (int pp = 0; pp < 4; pp++)
 #pragma unroll
-    for (int q = 0; q < 4; q++)
+    for (int q = 0; q < 2; q++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) acc[a][q][r] = 0.f;
+      for (int r = 0; r < 16; r++) acc[pp][q][r] = 0.f;
 
   // ---- main loop: two groups of four waves (one per SIMD each) run half a step out of phase.
   // While one group reads its fragments of a step from LDS (and issues its share of the loads for
   // later steps), the other group issues the 16 MFMAs of the step it read one phase earlier, so the
   // matrix cores of every SIMD always have a wave to serve.  Phases are separated by workgroup
-  // barriers; group 1 enters one barrier late and leaves one early.
+  // barriers; group 1 enters one barrier late, group 0 makes up for it after the loop.
   const int grp = wave >> 2;
 #pragma unroll
   for (int i = -C::kAheadMax; i < 0; i++) issue_step(i);
   wait_next_step_and_barrier(-1);
   if (grp == 1) wait_vmcnt_and_barrier<63>();
 
-#if FSW_DBG_TIMING == 4
-  const unsigned long long t_loop0 = __builtin_readcyclecounter();
-#endif
-#ifdef FSW_DBG_TIMING
-  unsigned long long* dbg = (unsigned long long*)p.c2;  // kDx/kDw leave c2 unused: harness passes a buffer
-  const bool dbg_on = (blockIdx.x == 8) && (lane == 0);
-#define FSW_STAMP(slot) do { if (kt >= 40 && kt < 48) { unsigned long long t_ = __builtin_readcyclecounter(); if (dbg_on) dbg[(wave * 8 + (kt - 40)) * 4 + (slot)] = t_; } } while (0)
-#else
-#define FSW_STAMP(slot) do {} while (0)
-#endif
   for (int kt = 0; kt < kt_total; kt++) {
     const FSW_LDS char* ra;
     const FSW_LDS char* rb;
@@ -264,135 +249,95 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
     if constexpr (B_KC) rb = lds_b + ((kt >> 1) % C::kAreasB) * kKcAreaBytes;
     else rb = lds_b + (kt & (kMcSlots - 1)) * kMcSlotBytes;
     const int half = kt & 1;
-#if FSW_DBG_TIMING == 1
-    FSW_STAMP(0);
-#endif
-    i16x8 fq[2][4], fp[2][2];
-#ifdef FSW_DBG_NO_LDSREAD
-    for (int ks = 0; ks < 2; ks++) { for (int q = 0; q < 4; q++) fq[ks][q] = (i16x8)(short)(kt + q); for (int a = 0; a < 2; a++) fp[ks][a] = (i16x8)(short)(kt + a); }
-    if (p.M < 0)
-#endif
+    i16x8 fq[2][2], fp[2][4];
 #pragma unroll
     for (int ks = 0; ks < 2; ks++) {
 #pragma unroll
-#ifdef FSW_DBG_HALFREADS
       for (int q = 0; q < 2; q++) {
-#else
-      for (int q = 0; q < 4; q++) {
-#endif
-        if constexpr (A_KC) fq[ks][q] = read_frag_kc(ra, wm * 128 + q * 32, half, ks, lane);
-        else fq[ks][q] = read_frag_mc(ra + wm * kMcPanelBytes, q, ks, lane);
+        if constexpr (A_KC) fq[ks][q] = read_frag_kc(ra, wm * 64 + q * 32, half, ks, lane);
+        else fq[ks][q] = read_frag_mc(ra + (wm >> 1) * kMcPanelBytes, (wm & 1) * 2 + q, ks, lane);
       }
 #pragma unroll
-#ifdef FSW_DBG_HALFREADS
-      for (int a = 0; a < 1; a++) {
-#else
-      for (int a = 0; a < 2; a++) {
-#endif
-        if constexpr (B_KC) fp[ks][a] = read_frag_kc(rb, wn * 64 + a * 32, half, ks, lane);
-        else fp[ks][a] = read_frag_mc(rb + a * kMcPanelBytes, wn, ks, lane);
+      for (int pp = 0; pp < 4; pp++) {
+        if constexpr (B_KC) fp[ks][pp] = read_frag_kc(rb, wn * 128 + pp * 32, half, ks, lane);
+        else fp[ks][pp] = read_frag_mc(rb + (pp >> 1) * kMcPanelBytes, wn * 2 + (pp & 1), ks, lane);
       }
     }
-#ifdef FSW_DBG_HALFREADS
-    // read only half of the A fragments and one B fragment; the rest are copies (timing experiment)
-    for (int ks = 0; ks < 2; ks++) { fq[ks][2] = fq[ks][0]; fq[ks][3] = fq[ks][1]; fp[ks][1] = fp[ks][0]; }
-#endif
-#ifndef FSW_DBG_NO_DMA
     issue_step(kt);
-#endif
-#if FSW_DBG_TIMING == 2
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    FSW_STAMP(1);
-#endif
     wait_next_step_and_barrier(kt);
-#if FSW_DBG_TIMING == 1 || FSW_DBG_TIMING == 3
-    FSW_STAMP(2);
-#endif
     __builtin_amdgcn_sched_barrier(0);
-#ifdef FSW_SETPRIO
-    __builtin_amdgcn_s_setprio(FSW_SETPRIO);
-#endif
 #pragma unroll
     for (int ks = 0; ks < 2; ks++)
-#ifdef FSW_MFMA_ORDER_AQ
 #pragma unroll
-      for (int a = 0; a < 2; a++)
+      for (int q = 0; q < 2; q++)
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-#else
-#pragma unroll
-      for (int q = 0; q < 4; q++)
-#pragma unroll
-        for (int a = 0; a < 2; a++) {
-#endif
-#ifdef FSW_DBG_NO_MFMA
-          { i16x8 t_ = fp[ks][a] ^ fq[ks][q]; i32x4 u_ = __builtin_bit_cast(i32x4, t_); acc[a][q][0] += __int_as_float(u_.x ^ u_.y ^ u_.z ^ u_.w); }
-#else
-          acc[a][q] = E::mfma(fp[ks][a], fq[ks][q], acc[a][q]);
-#endif
-        }
-#ifdef FSW_SETPRIO
-    __builtin_amdgcn_s_setprio(0);
-#endif
+        for (int pp = 0; pp < 4; pp++) acc[pp][q] = E::mfma(fp[ks][pp], fq[ks][q], acc[pp][q]);
     __builtin_amdgcn_sched_barrier(0);
-#if FSW_DBG_TIMING == 2 || FSW_DBG_TIMING == 3
-    FSW_STAMP(3);
-#endif
-    if (!(grp == 1 && kt == kt_total - 1)) wait_vmcnt_and_barrier<63>();
+    wait_vmcnt_and_barrier<63>();
   }
+  if (grp == 0) wait_vmcnt_and_barrier<63>();
+  // Every wave has passed its last read of the operand rings and every load has landed: LDS is free.
 
-#if FSW_DBG_TIMING == 4
-  { const unsigned long long t_loop1 = __builtin_readcyclecounter(); if (lane == 0 && (blockIdx.x & 255) == 8) { dbg[wave * 2] = t_loop1 - t_loop0; dbg[wave * 2 + 1] = kt_total; } }
-#endif
-  // ---- epilogue.  acc[a][q][r] of lane l is row  m0 + wm*128 + q*32 + (l & 31)  and column
-  //      cbase(a) + 8*(r >> 2) + 4*(l >> 5) + (r & 3): four consecutive columns per 8-byte store.
-#ifdef FSW_DBG_NO_STORE
-  if (p.M > 0 && acc[0][0][0] != 123.456f) return;
-#endif
-  const int mrow = m0 + wm * 128 + (lane & 31);
-  const int ncol_l = 4 * (lane >> 5);
+  // ---- epilogue.  acc[pp][q][r] of lane l is row  wm*64 + q*32 + (l & 31)  of the tile and column
+  // cbase(pp) + 8*(r >> 2) + 4*(l >> 5) + (r & 3).  Each wave owns 64 consecutive columns (128 bytes)
+  // per result row, so it transposes its 32 x 64 blocks through a private LDS patch and writes whole
+  // 128-byte lines: 8 rows x 128 bytes per store instruction instead of 32 rows x 16 bytes.
+  constexpr int kPatchPitch = 144;  // 128 + 16: keeps 16-byte alignment, spreads rows over banks
+  FSW_LDS char* patch = (FSW_LDS char*)smem + wave * (32 * kPatchPitch);
+  const int wr_off = (lane & 31) * kPatchPitch + (lane >> 5) * 8;       // + p*64 + r4*16
+  const int rd_off = (lane >> 3) * kPatchPitch + (lane & 7) * 16;       // + i*8*pitch
+  auto flush_patch = [&](unsigned short* dst, int col_base, int q) {
+    // rows q*32 + 8i + (lane >> 3), columns col_base + (lane & 7)*8 .. +8
 #pragma unroll
-  for (int q = 0; q < 4; q++) {
-    const int m = mrow + q * 32;
-    if (m >= p.M) continue;
+    for (int i = 0; i < 4; i++) {
+      const u32x4 v = *(const FSW_LDS u32x4*)(patch + rd_off + i * 8 * kPatchPitch);
+      const int m = m0 + wm * 64 + q * 32 + 8 * i + (lane >> 3);
+      const int n = col_base + (lane & 7) * 8;
+      if (m < p.M && n < p.N) *(u32x4*)(dst + (size_t)m * p.ldc + n) = v;
+    }
+  };
+  auto pack4 = [&](float a, float b, float c, float d) {
+    u32x2 v;
+    v.x = E::from_float(a) | ((unsigned)E::from_float(b) << 16);
+    v.y = E::from_float(c) | ((unsigned)E::from_float(d) << 16);
+    return v;
+  };
 #pragma unroll
-    for (int r4 = 0; r4 < 4; r4++) {
-      if constexpr (MODE == kFwd) {
-        const int n = n0 + wn * 32 + 8 * r4 + ncol_l;
-        if (n >= p.N) continue;
-        const size_t o = (size_t)m * p.ldc + n;
-        u32x2 vo, vg, vu;
-        unsigned short ho[4], hg[4], hu[4];
+  for (int q = 0; q < 2; q++) {
+    if constexpr (MODE == kFwd) {
+      // out = silu(g) * u, then g and u themselves (skipped when the caller passes no buffers for them)
 #pragma unroll
-        for (int e = 0; e < 4; e++) {
-          const float g = acc[0][q][r4 * 4 + e], u = acc[1][q][r4 * 4 + e];
-          ho[e] = E::from_float(silu_mul(g, u));
-          hg[e] = E::from_float(g);
-          hu[e] = E::from_float(u);
-        }
-        vo.x = ho[0] | ((unsigned)ho[1] << 16); vo.y = ho[2] | ((unsigned)ho[3] << 16);
-        *(u32x2*)((unsigned short*)p.c0 + o) = vo;
-        if (p.c1) {
-          vg.x = hg[0] | ((unsigned)hg[1] << 16); vg.y = hg[2] | ((unsigned)hg[3] << 16);
-          vu.x = hu[0] | ((unsigned)hu[1] << 16); vu.y = hu[2] | ((unsigned)hu[3] << 16);
-          *(u32x2*)((unsigned short*)p.c1 + o) = vg;
-          *(u32x2*)((unsigned short*)p.c2 + o) = vu;
-        }
-      } else {
+      for (int which = 0; which < 3; which++) {
+        if (which > 0 && p.c1 == nullptr) break;
 #pragma unroll
-        for (int a = 0; a < 2; a++) {
-          const int n = (MODE == kDx) ? n0 + wn * 64 + a * 32 + 8 * r4 + ncol_l
-                                      : n0 + wn * 32 + 8 * r4 + ncol_l;
-          if (n >= p.N) continue;
-          const size_t o = (size_t)m * p.ldc + n;
-          unsigned short h[4];
+        for (int pb = 0; pb < 2; pb++)
 #pragma unroll
-          for (int e = 0; e < 4; e++) h[e] = E::from_float(acc[a][q][r4 * 4 + e]);
-          u32x2 v;
-          v.x = h[0] | ((unsigned)h[1] << 16); v.y = h[2] | ((unsigned)h[3] << 16);
-          unsigned short* dst = (MODE == kDx || a == 0) ? (unsigned short*)p.c0 : (unsigned short*)p.c1;
-          *(u32x2*)(dst + o) = v;
-        }
+          for (int r4 = 0; r4 < 4; r4++) {
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              const float g = acc[pb][q][r4 * 4 + e], u = acc[2 + pb][q][r4 * 4 + e];
+              v[e] = which == 0 ? silu_mul(g, u) : (which == 1 ? g : u);
+            }
+            *(FSW_LDS u32x2*)(patch + wr_off + pb * 64 + r4 * 16) = pack4(v[0], v[1], v[2], v[3]);
+          }
+        unsigned short* dst = (unsigned short*)(which == 0 ? p.c0 : (which == 1 ? p.c1 : p.c2));
+        flush_patch(dst, n0 + wn * 64, q);
+      }
+    } else {
+      constexpr int kHalves = 2;  // kDx: two 64-column halves of one result; kDw: gate and up results
+#pragma unroll
+      for (int h = 0; h < kHalves; h++) {
+#pragma unroll
+        for (int pb = 0; pb < 2; pb++)
+#pragma unroll
+          for (int r4 = 0; r4 < 4; r4++) {
+            const f32x16& t = acc[2 * h + pb][q];
+            *(FSW_LDS u32x2*)(patch + wr_off + pb * 64 + r4 * 16) =
+                pack4(t[r4 * 4 + 0], t[r4 * 4 + 1], t[r4 * 4 + 2], t[r4 * 4 + 3]);
+          }
+        if constexpr (MODE == kDx) flush_patch((unsigned short*)p.c0, n0 + wn * 128 + h * 64, q);
+        else flush_patch((unsigned short*)(h == 0 ? p.c0 : p.c1), n0 + wn * 64, q);
       }
     }
   }

@@ -28,6 +28,10 @@ hipError_t launch_forward_fast(int dtype, const Problem& p, hipStream_t s);
 hipError_t launch_input_grad_fast(int dtype, const Problem& p, hipStream_t s);
 hipError_t launch_weight_grad_fast(int dtype, const Problem& p, hipStream_t s);
 
+// Weight-streaming forward for T <= 64 tokens (same eligibility as the tiled forward otherwise).
+bool skinny_forward_ok(const Problem& p);
+hipError_t launch_forward_skinny(int dtype, const Problem& p, hipStream_t s);
+
 // Any shape, any stride, 2-byte alignment: guarded element loads, same MFMA arithmetic.
 hipError_t launch_forward_generic(int dtype, const Problem& p, hipStream_t s);
 hipError_t launch_input_grad_generic(int dtype, const Problem& p, hipStream_t s);
