@@ -10,6 +10,7 @@ step), a roofline object for the dominant kernel measured live with GPU events o
 stream, and the eager fp32 PyTorch SwiGLU timed on this machine's host cores as CPU baseline.
 """
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -20,6 +21,16 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16/fp16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+
+# HBM-side bytes per launch (L2 <-> fabric reads + writes) of the three GEMM kernels at the C2 shape,
+# from the FETCH_SIZE / WRITE_SIZE counter passes summarised in profiles/gemm_kernels_c2_bf16.md
+# (FETCH_SIZE scaled by 2.0, WRITE_SIZE by 1.0 against a plain 1 GiB copy).  bench.py cannot run the
+# profiler itself; this table is refreshed whenever that profile is.
+PROFILED_TRAFFIC_BYTES = {
+    "forward_dual_gemm": (2 * 1179903 + 589824) * 1024,
+    "input_grad_dual_gemm": (2 * 1183105 + 65536) * 1024,
+    "weight_grad_dual_gemm": (2 * 1473863 + 196608) * 1024,
+}
 
 
 def parse():
@@ -127,7 +138,8 @@ def main():
         "peak": PEAK_BF16_TFLOPS,
         "unit": "TFLOP/s",
         "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
-        "traffic": None,
+        "traffic": PROFILED_TRAFFIC_BYTES.get(dominant),
+        "algorithmic_flop_per_launch": 4.0 * T * D * I,
     }
 
     result = {
@@ -150,6 +162,22 @@ def main():
         "roofline": roofline,
         "kernels": kernels,
     }
+
+    # ---- practical ceilings of this machine: register-only MFMA loop and a streaming read
+    if not args.no_extra:
+        sink = torch.zeros(4, device=dev, dtype=torch.float32)
+        ncu = torch.cuda.get_device_properties(dev).multi_processor_count
+        ceil = {}
+        for name, rnd in (("mfma_constant_operands_tflops", 0), ("mfma_normal_operands_tflops", 1)):
+            fl = ctypes.c_double(0.0)
+            run = lambda: _abi.check(L.fsw_probe_mfma(rnd, 20000, ncu, p(sink), stream, ctypes.byref(fl)))  # noqa: E731
+            ms = gpu_time_ms(run, iters=3, warmup=1)
+            ceil[name] = round(fl.value / ms / 1e9, 1)
+        big = torch.empty(1 << 31, device=dev, dtype=torch.uint8).fill_(1)
+        ms = gpu_time_ms(lambda: _abi.check(L.fsw_probe_stream_read(p(big), big.numel(), p(sink), stream)), iters=5, warmup=2)
+        ceil["hbm_stream_read_gbs"] = round(big.numel() / ms / 1e6, 1)
+        del big
+        result["measured_ceilings"] = ceil
 
     if args.calibrate_copy:
         src = torch.empty(1 << 30, device=dev, dtype=torch.uint8).fill_(1)

@@ -30,6 +30,8 @@ EXPORTED_SYMBOLS = (
     "fsw_elementwise_backward",
     "fsw_input_grad",
     "fsw_weight_grad",
+    "fsw_probe_mfma",
+    "fsw_probe_stream_read",
 )
 
 
@@ -96,6 +98,10 @@ def lib() -> ctypes.CDLL:
         L.fsw_input_grad.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, vp]
         L.fsw_weight_grad.restype = ci
         L.fsw_weight_grad.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, vp]
+        L.fsw_probe_mfma.restype = ci
+        L.fsw_probe_mfma.argtypes = [ci, ci, ci, vp, vp, ctypes.POINTER(ctypes.c_double)]
+        L.fsw_probe_stream_read.restype = ci
+        L.fsw_probe_stream_read.argtypes = [vp, i64, vp, vp]
         _lib = L
     return _lib
 

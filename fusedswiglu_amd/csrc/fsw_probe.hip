@@ -1,0 +1,75 @@
+// Two machine probes used by the benchmark to state practical ceilings next to the nominal peaks:
+// a register-only MFMA loop (no memory traffic at all) and a streaming read.  They only enqueue a
+// kernel; the caller times them with events on the same stream.
+#include "../../include/fusedswiglu.h"
+#include "fsw_common.hpp"
+
+namespace fsw {
+
+__device__ float probe_normal(unsigned i, unsigned seed) {
+  unsigned h = (i * 2654435761u) ^ seed;
+  h ^= h >> 15; h *= 0x2c1b3c6du; h ^= h >> 12; h *= 0x297a2d39u; h ^= h >> 15;
+  unsigned h2 = h * 0x9e3779b9u + 0x7f4a7c15u;
+  h2 ^= h2 >> 13; h2 *= 0x85ebca6bu; h2 ^= h2 >> 16;
+  const float u1 = ((h >> 8) + 1) * (1.0f / 16777217.0f), u2 = (h2 >> 8) * (1.0f / 16777216.0f);
+  return sqrtf(-2.f * logf(u1)) * cosf(6.2831853f * u2);
+}
+
+// 8 waves per workgroup, each issuing 8 independent 32x32x16 bf16 MFMAs per iteration.
+__global__ __launch_bounds__(512) void probe_mfma_kernel(float* sink, int iters, int random_operands) {
+  bf16x8 a[4], b[2];
+  for (int f = 0; f < 4; f++)
+    for (int j = 0; j < 8; j++)
+      a[f][j] = random_operands ? (__bf16)probe_normal(threadIdx.x * 64 + f * 8 + j + blockIdx.x * 77777, 1) : (__bf16)1.0f;
+  for (int f = 0; f < 2; f++)
+    for (int j = 0; j < 8; j++)
+      b[f][j] = random_operands ? (__bf16)(probe_normal(threadIdx.x * 64 + f * 8 + j + blockIdx.x * 33333, 2) * 0.015625f)
+                                : (__bf16)0.015625f;
+  f32x16 acc[2][4];
+  for (int x = 0; x < 2; x++)
+    for (int q = 0; q < 4; q++)
+      for (int r = 0; r < 16; r++) acc[x][q][r] = 0.f;
+  for (int it = 0; it < iters; it++) {
+#pragma unroll
+    for (int q = 0; q < 4; q++)
+#pragma unroll
+      for (int x = 0; x < 2; x++) acc[x][q] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[x], a[q], acc[x][q], 0, 0, 0);
+  }
+  float s = 0;
+  for (int x = 0; x < 2; x++)
+    for (int q = 0; q < 4; q++)
+      for (int r = 0; r < 16; r++) s += acc[x][q][r];
+  if (s == 12345.678f) sink[0] = s;  // keeps the loop alive; practically never true
+}
+
+__global__ __launch_bounds__(256) void probe_read_kernel(const u32x4* __restrict__ p, size_t n16, unsigned* sink) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  unsigned s = 0;
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  for (; i + 3 * stride < n16; i += 4 * stride) {
+    const u32x4 a = __builtin_nontemporal_load(p + i), b = __builtin_nontemporal_load(p + i + stride),
+                c = __builtin_nontemporal_load(p + i + 2 * stride), d = __builtin_nontemporal_load(p + i + 3 * stride);
+    s += a[0] ^ a[1] ^ a[2] ^ a[3] ^ b[0] ^ b[1] ^ b[2] ^ b[3] ^ c[0] ^ c[1] ^ c[2] ^ c[3] ^ d[0] ^ d[1] ^ d[2] ^ d[3];
+  }
+  for (; i < n16; i += stride) { const u32x4 a = p[i]; s += a[0] ^ a[1] ^ a[2] ^ a[3]; }
+  if (s == 0x12345678u) sink[0] = s;
+}
+
+}  // namespace fsw
+
+extern "C" {
+
+int fsw_probe_mfma(int random_operands, int iters, int workgroups, void* sink4, void* stream, double* flop_out) {
+  if (!sink4 || iters <= 0 || workgroups <= 0) return FSW_ERR_BAD_SHAPE;
+  fsw::probe_mfma_kernel<<<workgroups, 512, 0, (hipStream_t)stream>>>((float*)sink4, iters, random_operands);
+  if (flop_out) *flop_out = (double)workgroups * 8.0 * iters * 8.0 * 32768.0;
+  return hipGetLastError() == hipSuccess ? FSW_OK : FSW_ERR_LAUNCH;
+}
+
+int fsw_probe_stream_read(const void* buf, int64_t bytes, void* sink4, void* stream) {
+  if (!buf || !sink4 || bytes < 16 || ((uintptr_t)buf & 15)) return FSW_ERR_BAD_SHAPE;
+  fsw::probe_read_kernel<<<4096, 256, 0, (hipStream_t)stream>>>((const fsw::u32x4*)buf, (size_t)bytes / 16, (unsigned*)sink4);
+  return hipGetLastError() == hipSuccess ? FSW_OK : FSW_ERR_LAUNCH;
+}
+
+}  // extern "C"

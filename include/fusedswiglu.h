@@ -104,6 +104,17 @@ int fsw_weight_grad(const void* x, const void* grad_xw_up, const void* grad_xw_g
                     void* grad_w_up, void* grad_w_gate, int64_t T, int64_t D, int64_t I,
                     int64_t ldx, int64_t ldo, int64_t ld_dw, int dtype, void* stream);
 
+/*
+ * Machine probes for the benchmark harness (no counterpart in the reference).  Each call enqueues one
+ * kernel on `stream`; the caller times it with events.  sink4 is a 4-byte device scratch word.
+ * fsw_probe_mfma: `workgroups` x 8 waves issue `iters` x 8 back-to-back 32x32x16 bf16 MFMAs from
+ * registers (operands constant, or ~N(0,1) if random_operands != 0); *flop_out receives the flop count.
+ * fsw_probe_stream_read: grid-stride 16-byte reads of `bytes` bytes at buf (16-byte aligned).
+ */
+int fsw_probe_mfma(int random_operands, int iters, int workgroups, void* sink4, void* stream,
+                   double* flop_out);
+int fsw_probe_stream_read(const void* buf, int64_t bytes, void* sink4, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
