@@ -26,13 +26,8 @@ typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 struct BF16 {
   using vec8 = bf16x8;
   static FSW_DEV f32x16 mfma(i16x8 a, i16x8 b, f32x16 c) {
-#ifdef FSW_AGPR_ACC
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
-    return c;
-#else
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
                                                    __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-#endif
   }
   static FSW_DEV float to_float(unsigned short v) { return __uint_as_float((unsigned)v << 16); }
   // round-to-nearest-even; NaN stays NaN
@@ -83,14 +78,11 @@ FSW_DEV i32x4 make_rsrc(const void* base, unsigned num_records = 0x7fffffffu) {
 // (the LDS destination of a wave is contiguous by lane; lds_addr is wave-uniform).
 // Counted by vmcnt like any vector load; the compiler does not track it, so every consumer
 // must be fenced with wait_vmcnt<N>() + a workgroup barrier.
-#ifndef FSW_LOAD_MOD
-#define FSW_LOAD_MOD ""
-#endif
 FSW_DEV void load16_to_lds(i32x4 rsrc, unsigned voffset, unsigned lds_addr) {
   asm volatile(
       "s_mov_b32 m0, %0\n\t"
-      "s_nop 0\n\t"
-      "buffer_load_dwordx4 %1, %2, 0 offen " FSW_LOAD_MOD "lds"
+      "s_nop 3\n\t"  // M0 write -> LDS-DMA use, and any VALU-written descriptor SGPR -> VMEM read
+      "buffer_load_dwordx4 %1, %2, 0 offen lds"
       :
       : "s"(lds_addr), "v"(voffset), "s"(rsrc)
       : "memory");
@@ -99,27 +91,19 @@ FSW_DEV void load16_to_lds(i32x4 rsrc, unsigned voffset, unsigned lds_addr) {
 template <int N>
 FSW_DEV void wait_vmcnt_and_barrier() {
   static_assert(N >= 0 && N < 64, "vmcnt is 6 bits");
-#ifdef FSW_BARRIER_LGKM
-  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "n"(N) : "memory");
-#else
   // LDS reads issued before the barrier may still be in flight: their consumers carry their own
   // lgkmcnt waits, and no LDS slot is overwritten until a full step after it was last read
   asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" : : "n"(N) : "memory");
-#endif
 }
 
 // ---- LDS tile formats -------------------------------------------------------
-// Two formats, both for a k-step of BK = 32 elements of a 16-bit type.
-//
-// KC ("k-contiguous"): the operand is row-major with the reduction index innermost.  A tile is
-//   R rows x 64 bytes; the four 16-byte chunks of a row are stored at chunk position
-//   c ^ ((row >> 2) & 3).  Sixteen consecutive rows then cover all 64 LDS banks for a fixed
-//   logical chunk, so the ds_read_b128 fragment reads are conflict free.
-// MC ("m/n-contiguous"): the operand is row-major with the reduction index OUTERMOST.  A panel
+// The reduction advances kBK = 32 elements of a 16-bit type per step.
+// MC ("m/n-contiguous") panel: the operand is row-major with the reduction index OUTERMOST.  A panel
 //   is 32 k-rows x 256 bytes (128 columns); the four 64-byte blocks of a row are stored at block
 //   position b ^ (k & 3), so the four k-rows gathered by one ds_read_b64_tr_b16 hit disjoint banks.
+// The k-contiguous formats (rows of 128 or 64 bytes with XOR-swizzled 16-byte chunks) are described
+// where they are read: read_frag_kc in fsw_gemm.hpp, read_frag_x in fsw_skinny.hip.
 constexpr int kBK = 32;
-constexpr int kKcRowBytes = 64;
 constexpr int kMcRowBytes = 256;
 constexpr int kMcPanelBytes = kBK * kMcRowBytes;  // 8 KiB
 
