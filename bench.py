@@ -114,8 +114,8 @@ def main():
     calls = {
         "forward_dual_gemm": (lambda: _abi.check(L.fsw_swiglu_forward(p(xd), p(wgd), p(wud), p(out), p(g), p(u), T, D, I, D, I, I, 0, stream)), 4.0 * T * D * I),
         "elementwise_backward": (lambda: _abi.check(L.fsw_elementwise_backward(p(dout), p(g), p(u), p(dU), p(dG), T * I, 0, stream)), None),
-        "input_grad_dual_gemm": (lambda: _abi.check(L.fsw_input_grad(p(dG), p(dU), p(wgd), p(wud), p(dx), T, D, I, I, I, D, 0, stream)), 4.0 * T * D * I),
-        "weight_grad_dual_gemm": (lambda: _abi.check(L.fsw_weight_grad(p(xd), p(dU), p(dG), p(dWu), p(dWg), T, D, I, D, I, I, 0, stream)), 4.0 * T * D * I),
+        "input_grad_dual_gemm": (lambda: _abi.check(L.fsw_input_grad(p(dG), p(dU), p(wgd), p(wud), p(dx), T, D, I, I, I, D, None, 0, 0, stream)), 4.0 * T * D * I),
+        "weight_grad_dual_gemm": (lambda: _abi.check(L.fsw_weight_grad(p(xd), p(dU), p(dG), p(dWu), p(dWg), T, D, I, D, I, I, None, 0, 0, stream)), 4.0 * T * D * I),
     }
     kernels = {}
     for name, (fn, flop) in calls.items():

@@ -26,6 +26,7 @@ EXPORTED_SYMBOLS = (
     "fsw_last_error",
     "fsw_uses_tiled_kernel",
     "fsw_force_edge_kernels",
+    "fsw_workspace_bytes",
     "fsw_swiglu_forward",
     "fsw_elementwise_backward",
     "fsw_input_grad",
@@ -95,9 +96,11 @@ def lib() -> ctypes.CDLL:
         L.fsw_elementwise_backward.restype = ci
         L.fsw_elementwise_backward.argtypes = [vp, vp, vp, vp, vp, i64, ci, vp]
         L.fsw_input_grad.restype = ci
-        L.fsw_input_grad.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, vp]
+        L.fsw_input_grad.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, i64, ci, vp]
         L.fsw_weight_grad.restype = ci
-        L.fsw_weight_grad.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, vp]
+        L.fsw_weight_grad.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, i64, ci, vp]
+        L.fsw_workspace_bytes.restype = i64
+        L.fsw_workspace_bytes.argtypes = [ci, i64, i64, i64]
         L.fsw_probe_mfma.restype = ci
         L.fsw_probe_mfma.argtypes = [ci, ci, ci, vp, vp, ctypes.POINTER(ctypes.c_double)]
         L.fsw_probe_stream_read.restype = ci

@@ -83,6 +83,11 @@ int fsw_uses_tiled_kernel(int step, int64_t T, int64_t D, int64_t I, int64_t ldx
   }
 }
 
+int64_t fsw_workspace_bytes(int step, int64_t T, int64_t D, int64_t I) {
+  if (T <= 0 || D <= 0 || I <= 0) return 0;
+  return fsw::splitk_workspace_bytes(step, T, D, I);
+}
+
 int fsw_swiglu_forward(const void* x, const void* w_gate, const void* w_up, void* out,
                        void* xw_gate, void* xw_up, int64_t T, int64_t D, int64_t I, int64_t ldx,
                        int64_t ldw, int64_t ldo, int dtype, void* stream) {
@@ -122,7 +127,8 @@ int fsw_elementwise_backward(const void* grad_out, const void* xw_gate, const vo
 
 int fsw_input_grad(const void* grad_xw_gate, const void* grad_xw_up, const void* w_gate,
                    const void* w_up, void* grad_x, int64_t T, int64_t D, int64_t I, int64_t ldo,
-                   int64_t ldw, int64_t ld_dx, int dtype, void* stream) {
+                   int64_t ldw, int64_t ld_dx, void* workspace, int64_t workspace_bytes, int dtype,
+                   void* stream) {
   const char* fn = "fsw_input_grad";
   if (!grad_xw_gate || !grad_xw_up || !w_gate || !w_up || !grad_x)
     return fail(FSW_ERR_NULL_POINTER, "%s: all five arrays must be non-null", fn);
@@ -137,13 +143,17 @@ int fsw_input_grad(const void* grad_xw_gate, const void* grad_xw_up, const void*
   p.dG = grad_xw_gate; p.dU = grad_xw_up; p.wg = w_gate; p.wu = w_up; p.dx = grad_x;
   p.T = T; p.D = D; p.I = I; p.ldo = ldo; p.ldw = ldw; p.lddx = ld_dx;
   hipStream_t s = (hipStream_t)stream;
-  if (!g_force_edge.load() && fsw::fast_path_ok_input_grad(p)) return launched(fn, fsw::launch_input_grad_fast(dtype, p, s));
+  if (!g_force_edge.load() && fsw::fast_path_ok_input_grad(p)) {
+    const bool ws_ok = workspace && workspace_bytes > 0 && ((uintptr_t)workspace & 15) == 0;
+    return launched(fn, fsw::launch_input_grad_fast(dtype, p, s, ws_ok ? workspace : nullptr, ws_ok ? workspace_bytes : 0));
+  }
   return launched(fn, fsw::launch_input_grad_generic(dtype, p, s));
 }
 
 int fsw_weight_grad(const void* x, const void* grad_xw_up, const void* grad_xw_gate,
                     void* grad_w_up, void* grad_w_gate, int64_t T, int64_t D, int64_t I,
-                    int64_t ldx, int64_t ldo, int64_t ld_dw, int dtype, void* stream) {
+                    int64_t ldx, int64_t ldo, int64_t ld_dw, void* workspace, int64_t workspace_bytes,
+                    int dtype, void* stream) {
   const char* fn = "fsw_weight_grad";
   if (!x || !grad_xw_up || !grad_xw_gate || !grad_w_up || !grad_w_gate)
     return fail(FSW_ERR_NULL_POINTER, "%s: all five arrays must be non-null", fn);
@@ -158,7 +168,10 @@ int fsw_weight_grad(const void* x, const void* grad_xw_up, const void* grad_xw_g
   p.x = x; p.dG = grad_xw_gate; p.dU = grad_xw_up; p.dWg = grad_w_gate; p.dWu = grad_w_up;
   p.T = T; p.D = D; p.I = I; p.ldx = ldx; p.ldo = ldo; p.lddw = ld_dw;
   hipStream_t s = (hipStream_t)stream;
-  if (!g_force_edge.load() && fsw::fast_path_ok_weight_grad(p)) return launched(fn, fsw::launch_weight_grad_fast(dtype, p, s));
+  if (!g_force_edge.load() && fsw::fast_path_ok_weight_grad(p)) {
+    const bool ws_ok = workspace && workspace_bytes > 0 && ((uintptr_t)workspace & 15) == 0;
+    return launched(fn, fsw::launch_weight_grad_fast(dtype, p, s, ws_ok ? workspace : nullptr, ws_ok ? workspace_bytes : 0));
+  }
   return launched(fn, fsw::launch_weight_grad_generic(dtype, p, s));
 }
 

@@ -30,6 +30,11 @@ struct GemmParams {
   int M, N, K;     // GEMM view: kFwd (T,I,D)  kDx (T,D,I)  kDw (D,I,T)
   int lda, ldb, ldc;  // leading dimensions in elements
   int tiles_m, tiles_n, group_m;
+  // split-K (kDx, kDw on small problems): `splits` workgroups per tile each reduce `steps_per_split`
+  // steps (even) and store an fp32 partial tile to ws[split][M][N] (second result: + splits*M*N);
+  // fsw_splitk_reduce_kernel adds the partials in a fixed order.  splits == 1: results go to c0/c1.
+  float* ws;
+  int splits, steps_per_split;
 };
 
 constexpr int kThreads = 512;
@@ -141,13 +146,18 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;  // 4 waves along M x 2 along N
 
-  const TileCoord tc = xcd_tile_order(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m);
+  const int ntiles = p.tiles_m * p.tiles_n;
+  const int split = (MODE == kFwd) ? 0 : (int)(blockIdx.x / ntiles);
+  const TileCoord tc = xcd_tile_order((int)(blockIdx.x - split * ntiles), p.tiles_m, p.tiles_n, p.group_m);
   const int m0 = tc.tm * kTileM;
   const int n0 = tc.tn * TN;
 
   // steps per pass; kDx makes two passes (dG.Wg^T then dU.Wu^T) and keeps pairs of steps inside a pass
   const int kt1 = (MODE == kDx) ? (((p.K + kBK - 1) / kBK + 1) & ~1) : (p.K + kBK - 1) / kBK;
-  const int kt_total = (MODE == kDx) ? 2 * kt1 : kt1;
+  const int kt_all = (MODE == kDx) ? 2 * kt1 : kt1;
+  // this workgroup reduces steps kbase .. kbase + kt_total - 1 (everything unless split-K is on)
+  const int kbase = split * p.steps_per_split;
+  const int kt_total = (MODE == kFwd) ? kt_all : min(p.steps_per_split, kt_all - kbase);
 
   const unsigned smem_a = (unsigned)(uintptr_t)(FSW_LDS char*)smem;
   const unsigned smem_b = smem_a + C::kBytesA;
@@ -164,8 +174,9 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
   // loads of the pair of steps (pr, pr+1) of a KC operand into area (pr/2) % areas
   auto issue_kc = [&](const KcLoader& L, int pr, int areas, unsigned lds_base) {
     if (pr < 0 || pr >= kt_total) return;
-    const int pass = (MODE == kDx && pr >= kt1) ? 1 : 0;
-    const int k0 = (pr - pass * kt1) * kBK;
+    const int apr = kbase + pr;  // absolute step
+    const int pass = (MODE == kDx && apr >= kt1) ? 1 : 0;
+    const int k0 = (apr - pass * kt1) * kBK;
     const i32x4 rs = make_rsrc((pass ? L.base1 : L.base0) + (size_t)k0 * 2);
     const unsigned dst = lds_base + (unsigned)((pr >> 1) % areas) * kKcAreaBytes + wave * 1024;
 #pragma unroll
@@ -177,12 +188,12 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
   // loads of step s of an MC operand into slot s % 4
   auto issue_mc = [&](const McLoader& L, int s, unsigned lds_base) {
     if (s < 0 || s >= kt_total) return;
-    const int k0 = s * kBK;
+    const int k0 = (kbase + s) * kBK;
     const unsigned dst = lds_base + (unsigned)(s & (kMcSlots - 1)) * kMcSlotBytes + wave * 1024;
 #pragma unroll
     for (int i = 0; i < 2; i++) {
       const unsigned off = (k0 < L.klim[i]) ? L.lane_off[i] : kOobOffset;
-      load16_to_lds(make_rsrc(L.base[i] + (size_t)s * L.kstep), off, dst + i * 8192);
+      load16_to_lds(make_rsrc(L.base[i] + (size_t)(kbase + s) * L.kstep), off, dst + i * 8192);
     }
   };
   // everything a wave issues during step i (i < 0: prologue).  The order fixes the vmcnt arithmetic below.
@@ -282,6 +293,30 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
   // cbase(pp) + 8*(r >> 2) + 4*(l >> 5) + (r & 3).  Each wave owns 64 consecutive columns (128 bytes)
   // per result row, so it transposes its 32 x 64 blocks through a private LDS patch and writes whole
   // 128-byte lines: 8 rows x 128 bytes per store instruction instead of 32 rows x 16 bytes.
+  if (MODE != kFwd && p.splits > 1) {
+    // fp32 partial tile, 16 bytes (4 consecutive columns) per lane and store
+    const size_t plane = (size_t)p.M * p.N;
+#pragma unroll
+    for (int q = 0; q < 2; q++) {
+      const int m = m0 + wm * 64 + q * 32 + (lane & 31);
+      if (m >= p.M) continue;
+#pragma unroll
+      for (int pp = 0; pp < 4; pp++)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; r4++) {
+          const int ncol = 8 * r4 + 4 * (lane >> 5);
+          const int n = (MODE == kDx) ? n0 + wn * 128 + pp * 32 + ncol : n0 + wn * 64 + (pp & 1) * 32 + ncol;
+          if (n >= p.N) continue;
+          const size_t which = (MODE == kDx) ? 0 : (size_t)(pp >> 1);
+          float* dst = p.ws + (which * p.splits + split) * plane + (size_t)m * p.N + n;
+          f32x4 v;
+          v.x = acc[pp][q][r4 * 4 + 0]; v.y = acc[pp][q][r4 * 4 + 1];
+          v.z = acc[pp][q][r4 * 4 + 2]; v.w = acc[pp][q][r4 * 4 + 3];
+          *(f32x4*)dst = v;
+        }
+    }
+    return;
+  }
   constexpr int kPatchPitch = 144;  // 128 + 16: keeps 16-byte alignment, spreads rows over banks
   FSW_LDS char* patch = (FSW_LDS char*)smem + wave * (32 * kPatchPitch);
   const int wr_off = (lane & 31) * kPatchPitch + (lane >> 5) * 8;       // + p*64 + r4*16
@@ -341,6 +376,24 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
       }
     }
   }
+}
+
+// out[i] = round(sum over s of ws[s][i]), i < n, fixed order: deterministic.  n is a multiple of 4.
+template <typename E>
+__global__ __launch_bounds__(256) void fsw_splitk_reduce_kernel(const float* __restrict__ ws, unsigned short* __restrict__ out,
+                                                                size_t n, int splits, int N, int ldc) {
+  const size_t i4 = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (i4 >= n) return;
+  f32x4 a = *(const f32x4*)(ws + i4);
+  for (int s = 1; s < splits; s++) {
+    const f32x4 b = *(const f32x4*)(ws + (size_t)s * n + i4);
+    a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+  }
+  const size_t m = i4 / (size_t)N, c = i4 - m * (size_t)N;
+  u32x2 v;
+  v.x = E::from_float(a.x) | ((unsigned)E::from_float(a.y) << 16);
+  v.y = E::from_float(a.z) | ((unsigned)E::from_float(a.w) << 16);
+  *(u32x2*)(out + m * (size_t)ldc + c) = v;
 }
 
 }  // namespace fsw

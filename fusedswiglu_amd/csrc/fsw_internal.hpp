@@ -25,8 +25,10 @@ bool fast_path_ok_forward(const Problem& p);
 bool fast_path_ok_input_grad(const Problem& p);
 bool fast_path_ok_weight_grad(const Problem& p);
 hipError_t launch_forward_fast(int dtype, const Problem& p, hipStream_t s);
-hipError_t launch_input_grad_fast(int dtype, const Problem& p, hipStream_t s);
-hipError_t launch_weight_grad_fast(int dtype, const Problem& p, hipStream_t s);
+hipError_t launch_input_grad_fast(int dtype, const Problem& p, hipStream_t s, void* ws, long long ws_bytes);
+hipError_t launch_weight_grad_fast(int dtype, const Problem& p, hipStream_t s, void* ws, long long ws_bytes);
+// Bytes of fp32 scratch that let small input-grad (step 1) / weight-grad (step 2) problems split their reduction.
+long long splitk_workspace_bytes(int step, long long T, long long D, long long I);
 
 // Weight-streaming forward for T <= 64 tokens (same eligibility as the tiled forward otherwise).
 bool skinny_forward_ok(const Problem& p);

@@ -27,16 +27,89 @@ bool fast_path_ok_weight_grad(const Problem& p) {
          al16(p.dU) && al16(p.dWg) && al16(p.dWu);
 }
 
+// Split-K plan for a GEMM with `tiles` output tiles and `steps` reduction steps: few tiles and a long
+// reduction leave most of the 256 CUs idle, so several workgroups share a tile.  Returns 1 (no split)
+// when the tiles already fill the chip or the workspace is missing/too small.
+struct SplitPlan { int splits, steps_per_split; };
+// Estimated time (microseconds) of running `tiles * s` workgroups, each reducing 1/s of `steps` steps,
+// on 256 CUs: whole rounds of 256 workgroups at ~1 us per step, plus writing and re-reading the fp32
+// partial tiles at ~4 TB/s when s > 1.
+static double split_cost_us(long long tiles, int steps, int s, double result_elems) {
+  const long long wgs = tiles * s;
+  const double rounds = (double)((wgs + 255) / 256);
+  const double compute = rounds * ((double)steps / s + 6.0) * 0.96;  // + pipeline fill/epilogue per workgroup
+  const double partials = s > 1 ? 2.0 * s * result_elems * 4.0 / 4.0e6 : 0.0;
+  return compute + partials;
+}
+static SplitPlan plan_split_unbounded(long long tiles, int steps, long long M, long long N, int results) {
+  SplitPlan pl{1, steps};
+  if (tiles >= 1024 || steps < 32) return pl;
+  const double elems = (double)M * (double)N * results;
+  int best = 1;
+  double best_cost = split_cost_us(tiles, steps, 1, elems);
+  const int max_s = steps / 16 < 64 ? steps / 16 : 64;  // at least 16 steps per workgroup
+  for (int s = 2; s <= max_s; s++) {
+    const double c = split_cost_us(tiles, steps, s, elems);
+    if (c < best_cost * 0.95) { best_cost = c; best = s; }
+  }
+  if (best == 1) return pl;
+  int sps = (steps + best - 1) / best;
+  sps = (sps + 1) & ~1;                                  // pairs of steps stay together
+  pl.steps_per_split = sps;
+  pl.splits = (steps + sps - 1) / sps;
+  return pl;
+}
+static SplitPlan plan_split(long long tiles, int steps, long long M, long long N, int results,
+                            const void* ws, long long ws_bytes) {
+  SplitPlan pl = plan_split_unbounded(tiles, steps, M, N, results);
+  if (pl.splits > 1 && (!ws || (long long)pl.splits * M * N * 4 * results > ws_bytes)) return SplitPlan{1, steps};
+  return pl;
+}
+static int steps_of(int mode, long long K) {
+  int steps = (int)((K + kBK - 1) / kBK);
+  return mode == kDx ? 2 * ((steps + 1) & ~1) : steps;
+}
+
+long long splitk_workspace_bytes(int step, long long T, long long D, long long I) {
+  if (step == 1) {  // input_grad: result [T, D], reduction over 2*I
+    const long long tiles = ((T + kTileM - 1) / kTileM) * ((D + 255) / 256);
+    const SplitPlan pl = plan_split_unbounded(tiles, steps_of(kDx, I), T, D, 1);
+    return pl.splits > 1 ? (long long)pl.splits * T * D * 4 : 0;
+  }
+  if (step == 2) {  // weight_grad: results 2 x [D, I], reduction over T
+    const long long tiles = ((D + kTileM - 1) / kTileM) * ((I + 127) / 128);
+    const SplitPlan pl = plan_split_unbounded(tiles, steps_of(kDw, T), D, I, 2);
+    return pl.splits > 1 ? (long long)pl.splits * D * I * 4 * 2 : 0;
+  }
+  return 0;
+}
+
 template <int MODE>
-static hipError_t launch(int dtype, GemmParams g, hipStream_t s) {
+static hipError_t launch(int dtype, GemmParams g, hipStream_t s, void* ws = nullptr, long long ws_bytes = 0) {
   constexpr int TN = Cfg<MODE>::kTileN;
   g.tiles_m = (g.M + kTileM - 1) / kTileM;
   g.tiles_n = (g.N + TN - 1) / TN;
   g.group_m = 8;
   const long long tiles = (long long)g.tiles_m * g.tiles_n;
-  if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
-  if (dtype == kDtypeBF16) fsw_gemm_kernel<BF16, MODE><<<(unsigned)tiles, kThreads, 0, s>>>(g);
-  else fsw_gemm_kernel<FP16, MODE><<<(unsigned)tiles, kThreads, 0, s>>>(g);
+  const int steps = steps_of(MODE, g.K);
+  const int results = (MODE == kDw) ? 2 : 1;
+  const SplitPlan pl = (MODE == kFwd) ? SplitPlan{1, steps}
+                                      : plan_split(tiles, steps, g.M, g.N, results, ws, ws_bytes);
+  g.ws = (float*)ws; g.splits = pl.splits; g.steps_per_split = pl.steps_per_split;
+  const long long grid = tiles * pl.splits;
+  if (grid > 0x7fffffffLL) return hipErrorInvalidValue;
+  if (dtype == kDtypeBF16) fsw_gemm_kernel<BF16, MODE><<<(unsigned)grid, kThreads, 0, s>>>(g);
+  else fsw_gemm_kernel<FP16, MODE><<<(unsigned)grid, kThreads, 0, s>>>(g);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess || pl.splits == 1) return e;
+  const size_t n = (size_t)g.M * g.N;
+  const unsigned blocks = (unsigned)((n / 4 + 255) / 256);
+  for (int r = 0; r < results; r++) {
+    const float* src = (const float*)ws + (size_t)r * pl.splits * n;
+    unsigned short* dst = (unsigned short*)(r == 0 ? g.c0 : g.c1);
+    if (dtype == kDtypeBF16) fsw_splitk_reduce_kernel<BF16><<<blocks, 256, 0, s>>>(src, dst, n, pl.splits, g.N, g.ldc);
+    else fsw_splitk_reduce_kernel<FP16><<<blocks, 256, 0, s>>>(src, dst, n, pl.splits, g.N, g.ldc);
+  }
   return hipGetLastError();
 }
 
@@ -48,20 +121,20 @@ hipError_t launch_forward_fast(int dtype, const Problem& p, hipStream_t s) {
   return launch<kFwd>(dtype, g, s);
 }
 
-hipError_t launch_input_grad_fast(int dtype, const Problem& p, hipStream_t s) {
+hipError_t launch_input_grad_fast(int dtype, const Problem& p, hipStream_t s, void* ws, long long ws_bytes) {
   GemmParams g{};
   g.a0 = p.dG; g.a1 = p.dU; g.b0 = p.wg; g.b1 = p.wu; g.c0 = p.dx;
   g.M = (int)p.T; g.N = (int)p.D; g.K = (int)p.I;
   g.lda = (int)p.ldo; g.ldb = (int)p.ldw; g.ldc = (int)p.lddx;
-  return launch<kDx>(dtype, g, s);
+  return launch<kDx>(dtype, g, s, ws, ws_bytes);
 }
 
-hipError_t launch_weight_grad_fast(int dtype, const Problem& p, hipStream_t s) {
+hipError_t launch_weight_grad_fast(int dtype, const Problem& p, hipStream_t s, void* ws, long long ws_bytes) {
   GemmParams g{};
   g.a0 = p.x; g.b0 = p.dG; g.b1 = p.dU; g.c0 = p.dWg; g.c1 = p.dWu;
   g.M = (int)p.D; g.N = (int)p.I; g.K = (int)p.T;
   g.lda = (int)p.ldx; g.ldb = (int)p.ldo; g.ldc = (int)p.lddw;
-  return launch<kDw>(dtype, g, s);
+  return launch<kDw>(dtype, g, s, ws, ws_bytes);
 }
 
 }  // namespace fsw

@@ -50,6 +50,15 @@ def _rows(t: torch.Tensor) -> torch.Tensor:
     return t2
 
 
+def _workspace(step: int, T: int, D: int, I: int, dev: torch.device):
+    """(tensor or None, bytes) of fp32 scratch that lets a small gradient GEMM split its reduction
+    over several workgroups; the library says how much it wants (0 for problems that fill the chip)."""
+    nbytes = int(_abi.lib().fsw_workspace_bytes(step, T, D, I))
+    if nbytes <= 0:
+        return None, 0
+    return torch.empty(nbytes, device=dev, dtype=torch.uint8), nbytes
+
+
 def _ld(t2: torch.Tensor) -> int:
     return t2.stride(0) if t2.shape[0] > 1 else t2.shape[1]
 
@@ -126,9 +135,11 @@ def fused_input_grad(grad_xw_gate: torch.Tensor, grad_xw_up: torch.Tensor, w_gat
     T = dg.shape[0]
     grad_x = torch.empty(tuple(grad_xw_gate.shape[:-1]) + (D,), device=dev, dtype=dtype)
     with torch.cuda.device(dev):
+        ws, ws_bytes = _workspace(_abi.STEP_INPUT_GRAD, T, D, I, dev)
         _abi.check(_abi.lib().fsw_input_grad(
             dg.data_ptr(), du.data_ptr(), wg.data_ptr(), wu.data_ptr(), grad_x.data_ptr(),
-            T, D, I, _ld(dg), _ld(wg), D, _DTYPE_CODE[dtype], _stream_ptr(dev)))
+            T, D, I, _ld(dg), _ld(wg), D, ws.data_ptr() if ws is not None else None, ws_bytes,
+            _DTYPE_CODE[dtype], _stream_ptr(dev)))
     return grad_x
 
 
@@ -150,9 +161,11 @@ def fused_weight_grad(x: torch.Tensor, grad_xw_up: torch.Tensor, grad_xw_gate: t
     grad_w_up = torch.empty((D, I), device=dev, dtype=dtype)
     grad_w_gate = torch.empty((D, I), device=dev, dtype=dtype)
     with torch.cuda.device(dev):
+        ws, ws_bytes = _workspace(_abi.STEP_WEIGHT_GRAD, T, D, I, dev)
         _abi.check(_abi.lib().fsw_weight_grad(
             x2.data_ptr(), du.data_ptr(), dg.data_ptr(), grad_w_up.data_ptr(), grad_w_gate.data_ptr(),
-            T, D, I, _ld(x2), _ld(du), I, _DTYPE_CODE[dtype], _stream_ptr(dev)))
+            T, D, I, _ld(x2), _ld(du), I, ws.data_ptr() if ws is not None else None, ws_bytes,
+            _DTYPE_CODE[dtype], _stream_ptr(dev)))
     return grad_w_up, grad_w_gate
 
 

@@ -85,13 +85,24 @@ int fsw_elementwise_backward(const void* grad_out, const void* xw_gate, const vo
                              void* stream);
 
 /*
+ * Optional scratch for the two gradient GEMMs.  When a problem has too few output tiles to fill the
+ * chip (small d_model), several workgroups split the reduction of one tile, write fp32 partial
+ * tiles to `workspace` (device memory owned by the caller, 16-byte aligned, contents irrelevant) and
+ * a second kernel adds them in a fixed order.  fsw_workspace_bytes gives a sufficient size for
+ * step 1 (input_grad) or 2 (weight_grad); with workspace == NULL or a smaller size the call still
+ * works, just without (or with a smaller) split.  Large problems never touch the workspace.
+ */
+int64_t fsw_workspace_bytes(int step, int64_t T, int64_t D, int64_t I);
+
+/*
  * Input gradient: grad_x = grad_xw_gate Wg^T + grad_xw_up Wu^T, one kernel, one accumulator.
  * Replaces the two torch matmuls and the add at fused_swiglu/swiglu.py:45.
  *   grad_xw_gate, grad_xw_up [T,I] (ldo)   w_gate, w_up [D,I] (ldw)   grad_x [T,D] (ld_dx)
  */
 int fsw_input_grad(const void* grad_xw_gate, const void* grad_xw_up, const void* w_gate,
                    const void* w_up, void* grad_x, int64_t T, int64_t D, int64_t I, int64_t ldo,
-                   int64_t ldw, int64_t ld_dx, int dtype, void* stream);
+                   int64_t ldw, int64_t ld_dx, void* workspace, int64_t workspace_bytes, int dtype,
+                   void* stream);
 
 /*
  * Weight gradients: grad_w_gate = x^T grad_xw_gate, grad_w_up = x^T grad_xw_up, reduced over
@@ -102,7 +113,8 @@ int fsw_input_grad(const void* grad_xw_gate, const void* grad_xw_up, const void*
  */
 int fsw_weight_grad(const void* x, const void* grad_xw_up, const void* grad_xw_gate,
                     void* grad_w_up, void* grad_w_gate, int64_t T, int64_t D, int64_t I,
-                    int64_t ldx, int64_t ldo, int64_t ld_dw, int dtype, void* stream);
+                    int64_t ldx, int64_t ldo, int64_t ld_dw, void* workspace, int64_t workspace_bytes,
+                    int dtype, void* stream);
 
 /*
  * Machine probes for the benchmark harness (no counterpart in the reference).  Each call enqueues one

@@ -64,13 +64,19 @@ def test_backward_validation(L):
     assert e(P, P, P, P, P, 0, 0, None) == 3
     assert e(P, P, P, P, P, 8, 2, None) == 2
     dx = L.fsw_input_grad
-    assert dx(P, P, P, P, None, 8, 8, 8, 8, 8, 8, 0, None) == 1
-    assert dx(P, P, P, P, P, 8, 8, 8, 8, 8, 4, 0, None) == 4  # ld_dx < D
-    assert dx(P, P, P, P, P, 8, 8, 0, 8, 8, 8, 0, None) == 3
+    assert dx(P, P, P, P, None, 8, 8, 8, 8, 8, 8, None, 0, 0, None) == 1
+    assert dx(P, P, P, P, P, 8, 8, 8, 8, 8, 4, None, 0, 0, None) == 4  # ld_dx < D
+    assert dx(P, P, P, P, P, 8, 8, 0, 8, 8, 8, None, 0, 0, None) == 3
     dw = L.fsw_weight_grad
-    assert dw(P, None, P, P, P, 8, 8, 8, 8, 8, 8, 1, None) == 1
-    assert dw(P, P, P, P, P, 8, 8, 8, 8, 8, 8, -3, None) == 2
-    assert dw(P, P, P, P, P, 8, 16, 8, 8, 8, 8, 1, None) == 4  # ldx < D
+    assert dw(P, None, P, P, P, 8, 8, 8, 8, 8, 8, None, 0, 1, None) == 1
+    assert dw(P, P, P, P, P, 8, 8, 8, 8, 8, 8, None, 0, -3, None) == 2
+    assert dw(P, P, P, P, P, 8, 16, 8, 8, 8, 8, None, 0, 1, None) == 4  # ldx < D
+    # small d_model: few output tiles, long reductions -> the library asks for split-K scratch
+    assert L.fsw_workspace_bytes(1, 8192, 256, 768) % (8192 * 256 * 4) == 0 and L.fsw_workspace_bytes(1, 8192, 256, 768) > 0
+    assert L.fsw_workspace_bytes(2, 8192, 256, 768) % (2 * 256 * 768 * 4) == 0 and L.fsw_workspace_bytes(2, 8192, 256, 768) > 0
+    # the headline shape fills the chip: no scratch
+    assert L.fsw_workspace_bytes(1, 8192, 4096, 12288) == 0 and L.fsw_workspace_bytes(2, 8192, 4096, 12288) == 0
+    assert L.fsw_workspace_bytes(0, 8192, 256, 768) == 0 and L.fsw_workspace_bytes(1, 0, 1, 1) == 0
 
 
 def test_kernel_selection_logic(L):

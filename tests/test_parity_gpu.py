@@ -62,6 +62,8 @@ SMALL = [
     (2, 33, 72, 65),       # I not a multiple of 8 -> edge-shape kernel
     (1, 257, 100, 130),    # nothing aligned
     (1, 1, 4096, 24),      # single token, deep reduction
+    (4, 512, 256, 768),    # few output tiles, long reductions: gradient GEMMs split their reduction
+    (4, 500, 264, 776),    # the same with ragged edges; dx's second pass starts inside a split
 ]
 
 
