@@ -144,10 +144,14 @@ def fused_input_grad(grad_xw_gate: torch.Tensor, grad_xw_up: torch.Tensor, w_gat
 
 
 def fused_weight_grad(x: torch.Tensor, grad_xw_up: torch.Tensor, grad_xw_gate: torch.Tensor,
-                      dtype: torch.dtype) -> Tuple[torch.Tensor, torch.Tensor]:
+                      dtype: torch.dtype,
+                      out: Optional[Tuple[torch.Tensor, torch.Tensor]] = None
+                      ) -> Tuple[torch.Tensor, torch.Tensor]:
     """(grad_w_up, grad_w_gate) = (x^T grad_xw_up, x^T grad_xw_gate), each [D, I], reduced over
     every token in fp32.  Same argument and return order as fused_bmm (kernels_bf16.py:385-412),
-    with the batch sum of swiglu.py:56-57 folded in."""
+    with the batch sum of swiglu.py:56-57 folded in.  `out` = (grad_w_up, grad_w_gate) lets the
+    caller supply the two result arrays, e.g. the halves of one packed [D, 2I] gradient; they must
+    have unit inner stride and the same row stride."""
     _require(grad_xw_up.shape == grad_xw_gate.shape, "gate/up gradient shapes differ")
     _require(x.shape[:-1] == grad_xw_up.shape[:-1],
              f"Dimension mismatch. x {tuple(x.shape)} vs gradients {tuple(grad_xw_up.shape)}")
@@ -158,13 +162,23 @@ def fused_weight_grad(x: torch.Tensor, grad_xw_up: torch.Tensor, grad_xw_gate: t
         dg, du = dg.contiguous(), du.contiguous()
     T, D = x2.shape
     I = du.shape[1]
-    grad_w_up = torch.empty((D, I), device=dev, dtype=dtype)
-    grad_w_gate = torch.empty((D, I), device=dev, dtype=dtype)
+    if out is None:
+        grad_w_up = torch.empty((D, I), device=dev, dtype=dtype)
+        grad_w_gate = torch.empty((D, I), device=dev, dtype=dtype)
+    else:
+        grad_w_up, grad_w_gate = out
+        _require(tuple(grad_w_up.shape) == (D, I) and tuple(grad_w_gate.shape) == (D, I),
+                 f"weight-gradient outputs must be [{D}, {I}]")
+        _require(grad_w_up.dtype == dtype and grad_w_gate.dtype == dtype, f"Expected {dtype} tensors")
+        _check_device(x, grad_w_up, grad_w_gate)
+        _require(grad_w_up.stride(-1) == 1 and grad_w_gate.stride(-1) == 1 and _ld(grad_w_up) == _ld(grad_w_gate)
+                 and _ld(grad_w_up) >= I,
+                 "weight-gradient outputs need unit inner stride and equal row strides")
     with torch.cuda.device(dev):
         ws, ws_bytes = _workspace(_abi.STEP_WEIGHT_GRAD, T, D, I, dev)
         _abi.check(_abi.lib().fsw_weight_grad(
             x2.data_ptr(), du.data_ptr(), dg.data_ptr(), grad_w_up.data_ptr(), grad_w_gate.data_ptr(),
-            T, D, I, _ld(x2), _ld(du), I, ws.data_ptr() if ws is not None else None, ws_bytes,
+            T, D, I, _ld(x2), _ld(du), _ld(grad_w_up), ws.data_ptr() if ws is not None else None, ws_bytes,
             _DTYPE_CODE[dtype], _stream_ptr(dev)))
     return grad_w_up, grad_w_gate
 

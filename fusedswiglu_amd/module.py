@@ -1,0 +1,44 @@
+"""`nn.Module` wrapper around the fused SwiGLU path: the caller side of the operator boundary.
+
+The reference stops at `FusedSwiGLU.apply(x, w_gate, w_up)` and leaves holding the weights to the
+user (README.md:25-38).  `SwiGLU` owns them in the layout the kernels want ([d_model,
+d_intermediate], unit inner stride), initialised like the reference's tests draw them
+(N(0, 1)/sqrt(d_model), test_swiglu.py:30-35), either as two parameters or as one packed
+[d_model, 2*d_intermediate] parameter [w_gate | w_up]."""
+from __future__ import annotations
+
+import torch
+from torch import nn
+
+from . import ops
+
+
+class SwiGLU(nn.Module):
+    def __init__(self, d_model: int, d_intermediate: int, dtype: torch.dtype = torch.bfloat16,
+                 device=None, packed: bool = False):
+        super().__init__()
+        if dtype not in (torch.bfloat16, torch.float16):
+            raise ValueError(f"SwiGLU computes in bfloat16 or float16, got {dtype}")
+        self.d_model, self.d_intermediate, self.packed = d_model, d_intermediate, packed
+        kw = dict(device=device, dtype=dtype)
+        if packed:
+            self.w_gate_up = nn.Parameter(torch.empty(d_model, 2 * d_intermediate, **kw))
+        else:
+            self.w_gate = nn.Parameter(torch.empty(d_model, d_intermediate, **kw))
+            self.w_up = nn.Parameter(torch.empty(d_model, d_intermediate, **kw))
+        self.reset_parameters()
+
+    def reset_parameters(self) -> None:
+        std = self.d_model ** -0.5
+        for p in self.parameters():
+            if p.device.type != "meta":
+                nn.init.normal_(p, mean=0.0, std=std)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        dtype = next(self.parameters()).dtype
+        if self.packed:
+            return ops.swiglu_packed(x, self.w_gate_up, autocast_dtype=dtype)
+        return ops.swiglu(x, self.w_gate, self.w_up, autocast_dtype=dtype)
+
+    def extra_repr(self) -> str:
+        return f"d_model={self.d_model}, d_intermediate={self.d_intermediate}, packed={self.packed}"

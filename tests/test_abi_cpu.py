@@ -130,7 +130,9 @@ def test_python_boundary_errors_without_gpu():
 def test_package_exports():
     import fusedswiglu_amd
 
-    assert fusedswiglu_amd.__all__ == ["FusedSwiGLU", "FastAccumFusedSwiGLU"]
+    # the reference's two names first (fused_swiglu/__init__.py:1-2), then this build's additions
+    assert fusedswiglu_amd.__all__[:2] == ["FusedSwiGLU", "FastAccumFusedSwiGLU"]
+    assert set(fusedswiglu_amd.__all__[2:]) == {"swiglu", "swiglu_packed", "SwiGLU"}
     assert issubclass(FusedSwiGLU, torch.autograd.Function)
     assert issubclass(FastAccumFusedSwiGLU, torch.autograd.Function)
 

@@ -1,0 +1,45 @@
+"""Host-side checks of the torch.library operators and the nn.Module wrapper that need no GPU:
+shape inference of the fake implementations, parameter layout and initialisation, error behaviour."""
+import pytest
+import torch
+from torch._subclasses.fake_tensor import FakeTensorMode
+
+import fusedswiglu_amd as fsw
+from fusedswiglu_amd.kernels import kernels_bf16
+
+
+def test_fake_implementations_give_shapes_and_dtypes():
+    with FakeTensorMode():
+        for dtype in (torch.bfloat16, torch.float16):
+            x = torch.empty(2, 5, 16, dtype=dtype, device="cuda")
+            w = torch.empty(16, 24, dtype=dtype, device="cuda")
+            out, g, u = torch.ops.fusedswiglu_amd.swiglu_forward(x, w, w, True)
+            assert out.shape == g.shape == u.shape == (2, 5, 24) and out.dtype == dtype
+            out, g, u = torch.ops.fusedswiglu_amd.swiglu_forward(x, w, w, False)
+            assert out.shape == (2, 5, 24) and g.numel() == 0 and u.numel() == 0
+            dx, dwg, dwu = torch.ops.fusedswiglu_amd.swiglu_backward(out, x, w, w, out, out, True, True, False, False)
+            assert dx.shape == x.shape and dwg.shape == (16, 24) and dwu.numel() == 0
+            dx, dw, rest = torch.ops.fusedswiglu_amd.swiglu_backward(out, x, w, w, out, out, False, True, True, True)
+            assert dx.numel() == 0 and dw.shape == (16, 48) and rest.numel() == 0
+
+
+def test_module_parameters():
+    m = fsw.SwiGLU(64, 96)
+    assert m.w_gate.shape == m.w_up.shape == (64, 96) and m.w_gate.dtype == torch.bfloat16
+    # N(0, 1)/sqrt(d_model), as the reference's tests draw the weights (test_swiglu.py:30-35)
+    assert abs(float(m.w_gate.float().std()) * 8 - 1) < 0.1
+    p = fsw.SwiGLU(64, 96, dtype=torch.float16, packed=True)
+    assert p.w_gate_up.shape == (64, 192) and p.w_gate_up.dtype == torch.float16
+    assert [n for n, _ in p.named_parameters()] == ["w_gate_up"]
+    meta = fsw.SwiGLU(4096, 12288, device="meta")
+    assert meta.w_up.is_meta
+    with pytest.raises(ValueError):
+        fsw.SwiGLU(8, 8, dtype=torch.float32)
+
+
+def test_host_tensors_and_bad_shapes_are_rejected_before_any_launch():
+    m = fsw.SwiGLU(16, 24)
+    with pytest.raises(kernels_bf16.ShapeError, match="HIP GPU"):
+        m(torch.zeros(2, 16, dtype=torch.bfloat16))
+    with pytest.raises(kernels_bf16.ShapeError, match="packed weight"):
+        fsw.swiglu_packed(torch.zeros(2, 16), torch.zeros(16, 25))

@@ -235,6 +235,24 @@ def test_skinny_forward_full_width(oracle, M):
     _slice_check(oracle, torch.bfloat16, tx, twg, twu, None, out, None, None, None, n_rows=6)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("T,D,I", [(16, 256, 30720), (33, 264, 28672), (64, 512, 26632), (5, 136, 1800), (64, 128, 128)])
+def test_skinny_forward_column_blocks(oracle, dtype, T, D, I):
+    """Few tokens, many columns: the weight-streaming forward gives each workgroup a block of 128
+    columns; every column of out and of the saved pre-activations must land in its place, also in a
+    ragged last block and with more blocks than CUs."""
+    (x, wg, wu, _), (tx, twg, twu, _) = make(oracle, (1, T, D, I), dtype, seed=T)
+    out, g, u = KERN[dtype].fused_swiglu_fwd(tx, twg, twu)
+    torch.cuda.synchronize()
+    o_out, o_g, o_u = oracle.fused_swiglu_fwd(x, wg, wu)
+    tol = TOL[dtype]
+    assert oracle.rel_error(np64(out), o_out) < tol
+    assert oracle.rel_error(np64(g), o_g) < tol and oracle.rel_error(np64(u), o_u) < tol
+    # per-column check: a misplaced block would hide in a whole-array norm only if it were tiny
+    col_err = np.linalg.norm(np64(out)[0] - o_out[0], axis=0) / (np.linalg.norm(o_out[0], axis=0) + 1e-30)
+    assert col_err.max() < 20 * tol
+
+
 def test_large_config_slices(oracle):
     """x [8,4096,8192], W [8192,28672] (32768 tokens): forward + backward, checked on slices."""
     dtype, B, S, D, I = torch.bfloat16, 8, 4096, 8192, 28672
