@@ -30,7 +30,7 @@ hipError_t launch_weight_grad_fast(int dtype, const Problem& p, hipStream_t s, v
 // Bytes of fp32 scratch that let small input-grad (step 1) / weight-grad (step 2) problems split their reduction.
 long long splitk_workspace_bytes(int step, long long T, long long D, long long I);
 
-// Weight-streaming forward for T <= 64 tokens (same eligibility as the tiled forward otherwise).
+// Weight-streaming forward for T <= 128 tokens (same eligibility as the tiled forward otherwise).
 bool skinny_forward_ok(const Problem& p);
 hipError_t launch_forward_skinny(int dtype, const Problem& p, hipStream_t s);
 

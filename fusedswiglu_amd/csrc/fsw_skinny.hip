@@ -1,22 +1,29 @@
-// Weight-streaming forward for few tokens (T <= 64): out = silu(x Wg) * (x Wu).
+// Weight-streaming forward for few tokens (T <= 128): out = silu(x Wg) * (x Wu).
 // With so few rows the step is bound by reading Wg and Wu once from HBM, not by the MFMAs, so this
-// kernel is built around keeping many weight bytes in flight per CU: one workgroup of 4 waves owns
-// 128 columns of both weight matrices, walks the whole reduction in steps of 32, and keeps a ring of
-// 8 LDS stages (7 x 16 KiB of weights in flight) filled by direct global->LDS loads.  x (a few hundred
-// KiB, L2 resident) rides along in the same stages.  Each wave computes all BM rows x 32 columns of
-// the gate and the up product and applies silu(g)*u in registers.
+// kernel is built around keeping many weight bytes in flight per CU: one workgroup of 4 waves (one
+// per SIMD) owns 128 columns of both weight matrices, walks the whole reduction in steps of 32, and
+// keeps a ring of LDS stages (8 stages of 20 KiB for up to 64 rows, 6 of 24 KiB for 128)
+// filled by direct global->LDS loads.  x (a few MiB at most, L2 resident) rides along in the same
+// stages.  Each wave computes all BM rows x 32 columns of the gate and the up product and applies
+// silu(g)*u in registers.
 #include "fsw_gemm.hpp"
 #include "fsw_internal.hpp"
 
 namespace fsw {
 
-constexpr int kSkStages = 8;
 constexpr int kSkThreads = 256;
 
-// Every stage holds a 64-row x tile (4 KiB: one 1 KiB load per wave, rows beyond T zero-filled) and a
-// 16 KiB weight slot; BM only selects how many 32-row fragments are multiplied.
-constexpr int kSkABytes = 64 * 64;
-constexpr int kSkStage = kSkABytes + kMcSlotBytes;  // 20 KiB; 8 stages = 160 KiB
+// Every stage holds an x tile of max(BM, 64) rows x 64 bytes (1 KiB loads of 16 rows, one or more
+// per wave; rows beyond T zero-filled) and a 16 KiB weight slot.
+template <int BM>
+struct SkCfg {
+  static constexpr int kRowsX = BM < 64 ? 64 : BM;
+  static constexpr int kXBytes = kRowsX * 64;
+  static constexpr int kXLoads = kRowsX / 64;            // per wave and stage
+  static constexpr int kStage = kXBytes + kMcSlotBytes;  // 20 / 24 KiB
+  static constexpr int kStages = (160 * 1024) / kStage;  // 8 / 6
+  static constexpr int kPerStage = kXLoads + 4;          // loads a wave issues per stage
+};
 
 // x tile: BM rows x 64 bytes; chunk c of row r at position c ^ ((r >> 2) & 3) (see the MC/KC notes
 // in fsw_gemm.hpp; with 64-byte rows sixteen rows span the 64 banks when XOR-ed by (r >> 2)).
@@ -28,7 +35,9 @@ FSW_DEV i16x8 read_frag_x(const FSW_LDS char* a, int row_base, int ks, int lane)
 
 template <typename E, int BM>
 __global__ __launch_bounds__(kSkThreads) void fsw_skinny_forward_kernel(GemmParams p) {
+  using C = SkCfg<BM>;
   constexpr int NQ = BM / 32;
+  constexpr int kSkStages = C::kStages, kSkStage = C::kStage, kSkABytes = C::kXBytes;
   __shared__ __attribute__((aligned(1024))) char smem[kSkStages * kSkStage];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -37,14 +46,15 @@ __global__ __launch_bounds__(kSkThreads) void fsw_skinny_forward_kernel(GemmPara
   const unsigned smem_addr = (unsigned)(uintptr_t)(FSW_LDS char*)smem;
   const FSW_LDS char* smem_l = (const FSW_LDS char*)smem;
 
-  // x: wave w loads rows 16w .. 16w+15 (4 lanes x 16 bytes per row)
-  unsigned xa_off;
-  int xa_klim;
-  {
-    const int row = 16 * wave + (lane >> 2);
+  // x: load j of wave w covers rows 64j + 16w .. +15 (4 lanes x 16 bytes per row)
+  unsigned xa_off[C::kXLoads];
+  int xa_klim[C::kXLoads];
+#pragma unroll
+  for (int j = 0; j < C::kXLoads; j++) {
+    const int row = 64 * j + 16 * wave + (lane >> 2);
     const int c = (lane & 3) ^ ((lane >> 4) & 3);
-    xa_off = (unsigned)row * (unsigned)p.lda * 2u + c * 16u;
-    xa_klim = (row < p.M) ? p.K - c * 8 : -0x40000000;
+    xa_off[j] = (unsigned)row * (unsigned)p.lda * 2u + c * 16u;
+    xa_klim[j] = (row < p.M) ? p.K - c * 8 : -0x40000000;
   }
   // weights: 16 instructions per stage, 4 k-rows x 256 bytes each; instruction j -> panel j >> 3
   unsigned w_off[4];
@@ -60,14 +70,15 @@ __global__ __launch_bounds__(kSkThreads) void fsw_skinny_forward_kernel(GemmPara
     w_base[i] = (const char*)((j >> 3) ? p.b1 : p.b0) + (size_t)n0 * 2;
   }
   const size_t w_kstep = (size_t)kBK * p.ldb * 2;
-  constexpr int kPerStage = 1 + 4;  // loads a wave issues per stage
+  constexpr int kPerStage = C::kPerStage;
   auto issue = [&](int s) {
     if (s >= kt_total) return;
     const int k0 = s * kBK;
     const unsigned st = smem_addr + (unsigned)(s % kSkStages) * kSkStage;
-    {
-      const unsigned off = (k0 < xa_klim) ? xa_off : kOobOffset;
-      load16_to_lds(make_rsrc((const char*)p.a0 + (size_t)k0 * 2), off, st + wave * 1024);
+#pragma unroll
+    for (int j = 0; j < C::kXLoads; j++) {
+      const unsigned off = (k0 < xa_klim[j]) ? xa_off[j] : kOobOffset;
+      load16_to_lds(make_rsrc((const char*)p.a0 + (size_t)k0 * 2), off, st + j * 4096 + wave * 1024);
     }
 #pragma unroll
     for (int i = 0; i < 4; i++) {
@@ -91,9 +102,9 @@ __global__ __launch_bounds__(kSkThreads) void fsw_skinny_forward_kernel(GemmPara
     // stage kt landed?  up to kSkStages-2 younger stages may stay in flight
     const int younger = min(kt_total - 1 - kt, kSkStages - 2);
     switch (younger) {
-      case 6: wait_vmcnt_and_barrier<6 * kPerStage>(); break;
-      case 5: wait_vmcnt_and_barrier<5 * kPerStage>(); break;
-      case 4: wait_vmcnt_and_barrier<4 * kPerStage>(); break;
+      case 6: wait_vmcnt_and_barrier<(kSkStages > 7 ? 6 : 0) * kPerStage>(); break;
+      case 5: wait_vmcnt_and_barrier<(kSkStages > 6 ? 5 : 0) * kPerStage>(); break;
+      case 4: wait_vmcnt_and_barrier<(kSkStages > 5 ? 4 : 0) * kPerStage>(); break;
       case 3: wait_vmcnt_and_barrier<3 * kPerStage>(); break;
       case 2: wait_vmcnt_and_barrier<2 * kPerStage>(); break;
       case 1: wait_vmcnt_and_barrier<1 * kPerStage>(); break;
@@ -147,15 +158,20 @@ __global__ __launch_bounds__(kSkThreads) void fsw_skinny_forward_kernel(GemmPara
   }
 }
 
+// Beyond 128 rows the 64-byte x rows of this kernel (as many bytes per step as the weights by then)
+// cost more than the deeper ring gains: the tiled kernel takes over (measured at 256 rows: 300 vs 258 us).
+constexpr int kSkMaxRows = 128;
+
 template <typename E>
 static hipError_t launch_skinny_t(const GemmParams& g, hipStream_t s) {
   const unsigned tiles = (unsigned)((g.N + 127) / 128);
   if (g.M <= 32) fsw_skinny_forward_kernel<E, 32><<<tiles, kSkThreads, 0, s>>>(g);
-  else fsw_skinny_forward_kernel<E, 64><<<tiles, kSkThreads, 0, s>>>(g);
+  else if (g.M <= 64) fsw_skinny_forward_kernel<E, 64><<<tiles, kSkThreads, 0, s>>>(g);
+  else fsw_skinny_forward_kernel<E, 128><<<tiles, kSkThreads, 0, s>>>(g);
   return hipGetLastError();
 }
 
-bool skinny_forward_ok(const Problem& p) { return p.T <= 64 && fast_path_ok_forward(p); }
+bool skinny_forward_ok(const Problem& p) { return p.T <= kSkMaxRows && fast_path_ok_forward(p); }
 
 hipError_t launch_forward_skinny(int dtype, const Problem& p, hipStream_t s) {
   GemmParams g{};

@@ -236,10 +236,11 @@ def test_skinny_forward_full_width(oracle, M):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
-@pytest.mark.parametrize("T,D,I", [(16, 256, 30720), (33, 264, 28672), (64, 512, 26632), (5, 136, 1800), (64, 128, 128)])
+@pytest.mark.parametrize("T,D,I", [(16, 256, 30720), (33, 264, 28672), (64, 512, 26632), (5, 136, 1800), (64, 128, 128),
+                                   (100, 264, 1800), (128, 256, 1024), (200, 136, 776), (256, 512, 2056), (255, 4096, 136)])
 def test_skinny_forward_column_blocks(oracle, dtype, T, D, I):
-    """Few tokens, many columns: the weight-streaming forward gives each workgroup a block of 128
-    columns; every column of out and of the saved pre-activations must land in its place, also in a
+    """Up to 256 tokens: the weight-streaming forward (row-count variants 32/64/128/256) gives each
+    workgroup a block of 128 columns; every column of out and of the saved pre-activations must land in its place, also in a
     ragged last block and with more blocks than CUs."""
     (x, wg, wu, _), (tx, twg, twu, _) = make(oracle, (1, T, D, I), dtype, seed=T)
     out, g, u = KERN[dtype].fused_swiglu_fwd(tx, twg, twu)
