@@ -29,6 +29,11 @@ struct BF16 {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
                                                    __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
   }
+  // 16x16x32: half the accumulator traffic per flop of the 32x32x16 form (measurably less power)
+  static FSW_DEV f32x4 mfma16(i16x8 a, i16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
   static FSW_DEV float to_float(unsigned short v) { return __uint_as_float((unsigned)v << 16); }
   // round-to-nearest-even; NaN stays NaN
   static FSW_DEV unsigned short from_float(float f) {
@@ -39,6 +44,10 @@ struct FP16 {
   using vec8 = f16x8;
   static FSW_DEV f32x16 mfma(i16x8 a, i16x8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  static FSW_DEV f32x4 mfma16(i16x8 a, i16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a),
                                                   __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
   }
   static FSW_DEV float to_float(unsigned short v) {
@@ -100,7 +109,9 @@ FSW_DEV void wait_vmcnt_and_barrier() {
 // The reduction advances kBK = 32 elements of a 16-bit type per step.
 // MC ("m/n-contiguous") panel: the operand is row-major with the reduction index OUTERMOST.  A panel
 //   is 32 k-rows x 256 bytes (128 columns); the four 64-byte blocks of a row are stored at block
-//   position b ^ (k & 3), so the four k-rows gathered by one ds_read_b64_tr_b16 hit disjoint banks.
+//   position b ^ (k & 3), so the four k-rows gathered by one ds_read_b64_tr_b16 hit disjoint banks
+//   (the tiled kernel additionally swaps the 32-byte halves of every block on k-rows 8..15 and
+//   24..31, see read_frag_mc16).
 // The k-contiguous formats (rows of 128 or 64 bytes with XOR-swizzled 16-byte chunks) are described
 // where they are read: read_frag_kc in fsw_gemm.hpp, read_frag_x in fsw_skinny.hip.
 constexpr int kBK = 32;

@@ -66,22 +66,39 @@ struct Cfg {
 // ---- fragment reads -----------------------------------------------------------
 // KC area: 256 rows x 128 bytes; the 16-byte chunk c of row r sits at chunk position
 // c ^ ((r >> 1) & 7), so that 16 consecutive rows cover all 64 banks for a fixed c.
-// Lane l gets row (l & 31), k = half*32 + ks*16 + 8*(l >> 5) .. +8 in one ds_read_b128.
-FSW_DEV i16x8 read_frag_kc(const FSW_LDS char* area, int row_base, int half, int ks, int lane) {
-  const int row = row_base + (lane & 31);
-  const int chunk = (half * 4 + ks * 2 + (lane >> 5)) ^ ((lane >> 1) & 7);
+// 16x16x32 operand: lane l gets row (l & 15), k = half*32 + 8*(l >> 4) .. +8 in one ds_read_b128.
+FSW_DEV i16x8 read_frag_kc16(const FSW_LDS char* area, int row_base, int half, int lane) {
+  const int row = row_base + (lane & 15);
+  const int chunk = (half * 4 + (lane >> 4)) ^ ((lane >> 1) & 7);
   return *(const FSW_LDS i16x8*)(area + row * 128 + chunk * 16);
 }
 
-// MC panel: 32 k-rows x 256 bytes; the 64-byte block b of k-row k sits at block position b ^ (k & 3).
-// Two transposing reads.  Within each group of 16 lanes, lane j supplies the address of 4
-// consecutive columns (j & 3)*4.. of k-row (j >> 2); the hardware hands lane i the column i of
-// those four k-rows.  Lane groups 0/1 cover columns 0-15 / 16-31 of the 32-column fragment,
-// groups 2/3 the same columns 8 k-rows further on -- the MFMA operand layout.
+// MC panel of the weight-streaming kernel: 32 k-rows x 256 bytes; the 64-byte block b of k-row k sits
+// at block position b ^ (k & 3).  32x32x16 operand by two transposing reads.  Within each group of 16
+// lanes, lane j supplies the address of 4 consecutive columns (j & 3)*4.. of k-row (j >> 2); the
+// hardware hands lane i the column i of those four k-rows.  Lane groups 0/1 cover columns 0-15 /
+// 16-31 of the 32-column fragment, groups 2/3 the same columns 8 k-rows further on.
 FSW_DEV i16x8 read_frag_mc(const FSW_LDS char* panel, int block64, int ks, int lane) {
   const int grp = lane >> 4, j = lane & 15;
   const int krow = ks * 16 + 8 * (grp >> 1) + (j >> 2);
   const int byte = krow * kMcRowBytes + ((block64 ^ (j >> 2)) * 64) + ((grp & 1) * 16 + (j & 3) * 4) * 2;
+  i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FSW_LDS i16x4*)(panel + byte));
+  i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FSW_LDS i16x4*)(panel + byte + 4 * kMcRowBytes));
+  i16x8 r;
+  r.s0 = lo.x; r.s1 = lo.y; r.s2 = lo.z; r.s3 = lo.w;
+  r.s4 = hi.x; r.s5 = hi.y; r.s6 = hi.z; r.s7 = hi.w;
+  return r;
+}
+
+// MC panel of the tiled kernel: as above, and in k-rows with (k >> 3) odd the two 32-byte halves of
+// every 64-byte block are swapped.  16x16x32 operand (16 columns x 32 k-rows) by two transposing
+// reads: lane group g covers k-rows 8g .. 8g+7 (first read 8g..+3, second 8g+4..+7) of the same 16
+// columns, lane j of a group supplying columns (j & 3)*4.. of k-row (j >> 2).  Groups 0 and 1 (and 2
+// and 3) then sit in different 32-byte halves, so each half-wave touches every bank once.
+FSW_DEV i16x8 read_frag_mc16(const FSW_LDS char* panel, int frag16, int lane) {
+  const int grp = lane >> 4, j = lane & 15;
+  const int krow = 8 * grp + (j >> 2);
+  const int byte = krow * kMcRowBytes + (((frag16 >> 1) ^ (j >> 2)) * 64) + (((frag16 ^ grp) & 1) * 32) + (j & 3) * 8;
   i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FSW_LDS i16x4*)(panel + byte));
   i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FSW_LDS i16x4*)(panel + byte + 4 * kMcRowBytes));
   i16x8 r;
@@ -125,7 +142,8 @@ FSW_DEV void mc_setup(McLoader& L, const void* p_panel0, const void* p_panel1, i
   for (int i = 0; i < 2; i++) {
     const int j = wave + 8 * i;
     const int row = 4 * (j & 7) + (lane >> 4);
-    const int col = (((lane >> 2) & 3) ^ ((lane >> 4) & 3)) * 32 + (lane & 3) * 8;
+    // physical 16-byte chunk (lane & 15) of k-row `row` holds logical columns `col`.. (see read_frag_mc16)
+    const int col = (((lane >> 2) & 3) ^ (row & 3)) * 32 + ((((lane >> 1) ^ (row >> 3)) & 1) * 16) + (lane & 1) * 8;
     const int col0 = (j >> 3) ? col0_panel1 : col0_panel0;
     L.lane_off[i] = (unsigned)row * (unsigned)ld * 2u + col * 2u;
     L.klim[i] = (col0 + col < cols_total) ? K - row : -0x40000000;
@@ -230,20 +248,18 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
     }
   };
 
-  // acc[pp][q]: 32x32 block of rows wm*64 + q*32.. and column block pp of this wave:
-  //   kFwd/kDw  pp = 2*a + p: matrix a (gate | up), columns wn*64 + p*32..
-  //   kDx       columns wn*128 + pp*32..
-  f32x16 acc[4][2];
+  // acc[nb][mb]: 16x16 block of rows wm*64 + mb*16.. and 16-column block nb of this wave:
+  //   kFwd/kDw  nb = 4*a + c: matrix a (gate | up), columns wn*64 + c*16..
+  //   kDx       columns wn*128 + nb*16..
+  f32x4 acc[8][4];
 #pragma unroll
-  for (int pp = 0; pp < 4; pp++)
+  for (int nb = 0; nb < 8; nb++)
 #pragma unroll
-    for (int q = 0; q < 2; q++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) acc[pp][q][r] = 0.f;
+    for (int mb = 0; mb < 4; mb++) acc[nb][mb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   // ---- main loop: two groups of four waves (one per SIMD each) run half a step out of phase.
   // While one group reads its fragments of a step from LDS (and issues its share of the loads for
-  // later steps), the other group issues the 16 MFMAs of the step it read one phase earlier, so the
+  // later steps), the other group issues the 32 MFMAs of the step it read one phase earlier, so the
   // matrix cores of every SIMD always have a wave to serve.  Phases are separated by workgroup
   // barriers; group 1 enters one barrier late, group 0 makes up for it after the loop.
   const int grp = wave >> 2;
@@ -260,66 +276,60 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
     if constexpr (B_KC) rb = lds_b + ((kt >> 1) % C::kAreasB) * kKcAreaBytes;
     else rb = lds_b + (kt & (kMcSlots - 1)) * kMcSlotBytes;
     const int half = kt & 1;
-    i16x8 fq[2][2], fp[2][4];
+    i16x8 fq[4], fp[8];
 #pragma unroll
-    for (int ks = 0; ks < 2; ks++) {
+    for (int mb = 0; mb < 4; mb++) {
+      if constexpr (A_KC) fq[mb] = read_frag_kc16(ra, wm * 64 + mb * 16, half, lane);
+      else fq[mb] = read_frag_mc16(ra + (wm >> 1) * kMcPanelBytes, (wm & 1) * 4 + mb, lane);
+    }
 #pragma unroll
-      for (int q = 0; q < 2; q++) {
-        if constexpr (A_KC) fq[ks][q] = read_frag_kc(ra, wm * 64 + q * 32, half, ks, lane);
-        else fq[ks][q] = read_frag_mc(ra + (wm >> 1) * kMcPanelBytes, (wm & 1) * 2 + q, ks, lane);
-      }
-#pragma unroll
-      for (int pp = 0; pp < 4; pp++) {
-        if constexpr (B_KC) fp[ks][pp] = read_frag_kc(rb, wn * 128 + pp * 32, half, ks, lane);
-        else fp[ks][pp] = read_frag_mc(rb + (pp >> 1) * kMcPanelBytes, wn * 2 + (pp & 1), ks, lane);
-      }
+    for (int nb = 0; nb < 8; nb++) {
+      if constexpr (B_KC) fp[nb] = read_frag_kc16(rb, wn * 128 + nb * 16, half, lane);
+      else fp[nb] = read_frag_mc16(rb + (nb >> 2) * kMcPanelBytes, wn * 4 + (nb & 3), lane);
     }
     issue_step(kt);
     wait_next_step_and_barrier(kt);
     __builtin_amdgcn_sched_barrier(0);
+    // consecutive MFMAs share one operand (the m index snakes back and forth)
 #pragma unroll
-    for (int ks = 0; ks < 2; ks++)
+    for (int nb = 0; nb < 8; nb++)
 #pragma unroll
-      for (int q = 0; q < 2; q++)
-#pragma unroll
-        for (int pp = 0; pp < 4; pp++) acc[pp][q] = E::mfma(fp[ks][pp], fq[ks][q], acc[pp][q]);
+      for (int i = 0; i < 4; i++) {
+        const int mb = (nb & 1) ? 3 - i : i;
+        acc[nb][mb] = E::mfma16(fp[nb], fq[mb], acc[nb][mb]);
+      }
     __builtin_amdgcn_sched_barrier(0);
     wait_vmcnt_and_barrier<63>();
   }
   if (grp == 0) wait_vmcnt_and_barrier<63>();
   // Every wave has passed its last read of the operand rings and every load has landed: LDS is free.
 
-  // ---- epilogue.  acc[pp][q][r] of lane l is row  wm*64 + q*32 + (l & 31)  of the tile and column
-  // cbase(pp) + 8*(r >> 2) + 4*(l >> 5) + (r & 3).  Each wave owns 64 consecutive columns (128 bytes)
-  // per result row, so it transposes its 32 x 64 blocks through a private LDS patch and writes whole
-  // 128-byte lines: 8 rows x 128 bytes per store instruction instead of 32 rows x 16 bytes.
+  // ---- epilogue.  acc[nb][mb][r] of lane l is row  wm*64 + mb*16 + (l & 15)  of the tile and column
+  // cbase(nb) + 4*(l >> 4) + r.  Each wave owns 64 consecutive columns (128 bytes) per result row, so
+  // it transposes 32 rows x 64 columns at a time through a private LDS patch and writes whole 128-byte
+  // lines: 8 rows x 128 bytes per store instruction.
   if (MODE != kFwd && p.splits > 1) {
     // fp32 partial tile, 16 bytes (4 consecutive columns) per lane and store
     const size_t plane = (size_t)p.M * p.N;
 #pragma unroll
-    for (int q = 0; q < 2; q++) {
-      const int m = m0 + wm * 64 + q * 32 + (lane & 31);
+    for (int mb = 0; mb < 4; mb++) {
+      const int m = m0 + wm * 64 + mb * 16 + (lane & 15);
       if (m >= p.M) continue;
 #pragma unroll
-      for (int pp = 0; pp < 4; pp++)
-#pragma unroll
-        for (int r4 = 0; r4 < 4; r4++) {
-          const int ncol = 8 * r4 + 4 * (lane >> 5);
-          const int n = (MODE == kDx) ? n0 + wn * 128 + pp * 32 + ncol : n0 + wn * 64 + (pp & 1) * 32 + ncol;
-          if (n >= p.N) continue;
-          const size_t which = (MODE == kDx) ? 0 : (size_t)(pp >> 1);
-          float* dst = p.ws + (which * p.splits + split) * plane + (size_t)m * p.N + n;
-          f32x4 v;
-          v.x = acc[pp][q][r4 * 4 + 0]; v.y = acc[pp][q][r4 * 4 + 1];
-          v.z = acc[pp][q][r4 * 4 + 2]; v.w = acc[pp][q][r4 * 4 + 3];
-          *(f32x4*)dst = v;
-        }
+      for (int nb = 0; nb < 8; nb++) {
+        const int ncol = 4 * (lane >> 4);
+        const int n = (MODE == kDx) ? n0 + wn * 128 + nb * 16 + ncol : n0 + wn * 64 + (nb & 3) * 16 + ncol;
+        if (n >= p.N) continue;
+        const size_t which = (MODE == kDx) ? 0 : (size_t)(nb >> 2);
+        float* dst = p.ws + (which * p.splits + split) * plane + (size_t)m * p.N + n;
+        *(f32x4*)dst = acc[nb][mb];
+      }
     }
     return;
   }
   constexpr int kPatchPitch = 144;  // 128 + 16: keeps 16-byte alignment, spreads rows over banks
   FSW_LDS char* patch = (FSW_LDS char*)smem + wave * (32 * kPatchPitch);
-  const int wr_off = (lane & 31) * kPatchPitch + (lane >> 5) * 8;       // + p*64 + r4*16
+  const int wr_off = (lane & 15) * kPatchPitch + (lane >> 4) * 8;       // + mbl*16*pitch + c*32
   const int rd_off = (lane >> 3) * kPatchPitch + (lane & 7) * 16;       // + i*8*pitch
   auto flush_patch = [&](unsigned short* dst, int col_base, int q) {
     // rows q*32 + 8i + (lane >> 3), columns col_base + (lane & 7)*8 .. +8
@@ -338,23 +348,21 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
     return v;
   };
 #pragma unroll
-  for (int q = 0; q < 2; q++) {
+  for (int q = 0; q < 2; q++) {  // 32 rows of the wave's 64 at a time
     if constexpr (MODE == kFwd) {
       // out = silu(g) * u, then g and u themselves (skipped when the caller passes no buffers for them)
 #pragma unroll
       for (int which = 0; which < 3; which++) {
         if (which > 0 && p.c1 == nullptr) break;
 #pragma unroll
-        for (int pb = 0; pb < 2; pb++)
+        for (int mbl = 0; mbl < 2; mbl++)
 #pragma unroll
-          for (int r4 = 0; r4 < 4; r4++) {
+          for (int c = 0; c < 4; c++) {
+            const f32x4 g = acc[c][2 * q + mbl], u = acc[4 + c][2 * q + mbl];
             float v[4];
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-              const float g = acc[pb][q][r4 * 4 + e], u = acc[2 + pb][q][r4 * 4 + e];
-              v[e] = which == 0 ? silu_mul(g, u) : (which == 1 ? g : u);
-            }
-            *(FSW_LDS u32x2*)(patch + wr_off + pb * 64 + r4 * 16) = pack4(v[0], v[1], v[2], v[3]);
+            for (int e = 0; e < 4; e++) v[e] = which == 0 ? silu_mul(g[e], u[e]) : (which == 1 ? g[e] : u[e]);
+            *(FSW_LDS u32x2*)(patch + wr_off + mbl * 16 * kPatchPitch + c * 32) = pack4(v[0], v[1], v[2], v[3]);
           }
         unsigned short* dst = (unsigned short*)(which == 0 ? p.c0 : (which == 1 ? p.c1 : p.c2));
         flush_patch(dst, n0 + wn * 64, q);
@@ -364,12 +372,11 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
 #pragma unroll
       for (int h = 0; h < kHalves; h++) {
 #pragma unroll
-        for (int pb = 0; pb < 2; pb++)
+        for (int mbl = 0; mbl < 2; mbl++)
 #pragma unroll
-          for (int r4 = 0; r4 < 4; r4++) {
-            const f32x16& t = acc[2 * h + pb][q];
-            *(FSW_LDS u32x2*)(patch + wr_off + pb * 64 + r4 * 16) =
-                pack4(t[r4 * 4 + 0], t[r4 * 4 + 1], t[r4 * 4 + 2], t[r4 * 4 + 3]);
+          for (int c = 0; c < 4; c++) {
+            const f32x4 t = acc[4 * h + c][2 * q + mbl];
+            *(FSW_LDS u32x2*)(patch + wr_off + mbl * 16 * kPatchPitch + c * 32) = pack4(t[0], t[1], t[2], t[3]);
           }
         if constexpr (MODE == kDx) flush_patch((unsigned short*)p.c0, n0 + wn * 128 + h * 64, q);
         else flush_patch((unsigned short*)(h == 0 ? p.c0 : p.c1), n0 + wn * 64, q);
