@@ -29,6 +29,7 @@ EXPORTED_SYMBOLS = (
     "fsw_workspace_bytes",
     "fsw_swiglu_forward",
     "fsw_elementwise_backward",
+    "fsw_gating_grad_recompute",
     "fsw_input_grad",
     "fsw_weight_grad",
     "fsw_probe_mfma",
@@ -95,6 +96,8 @@ def lib() -> ctypes.CDLL:
         L.fsw_swiglu_forward.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, vp]
         L.fsw_elementwise_backward.restype = ci
         L.fsw_elementwise_backward.argtypes = [vp, vp, vp, vp, vp, i64, ci, vp]
+        L.fsw_gating_grad_recompute.restype = ci
+        L.fsw_gating_grad_recompute.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, vp]
         L.fsw_input_grad.restype = ci
         L.fsw_input_grad.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, i64, ci, vp]
         L.fsw_weight_grad.restype = ci

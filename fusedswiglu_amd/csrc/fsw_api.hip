@@ -76,7 +76,8 @@ int fsw_uses_tiled_kernel(int step, int64_t T, int64_t D, int64_t I, int64_t ldx
   p.out = p.g = p.u = p.dx = p.dWg = p.dWu = (void*)ptr;
   p.T = T; p.D = D; p.I = I; p.ldx = ldx; p.ldw = ldw; p.ldo = ldo; p.lddx = ld_grad; p.lddw = ld_grad;
   switch (step) {
-    case 0: return fsw::fast_path_ok_forward(p) ? 1 : 0;
+    case 0:
+    case 3: return fsw::fast_path_ok_forward(p) ? 1 : 0;
     case 1: return fsw::fast_path_ok_input_grad(p) ? 1 : 0;
     case 2: return fsw::fast_path_ok_weight_grad(p) ? 1 : 0;
     default: return 0;
@@ -107,6 +108,28 @@ int fsw_swiglu_forward(const void* x, const void* w_gate, const void* w_up, void
   p.T = T; p.D = D; p.I = I; p.ldx = ldx; p.ldw = ldw; p.ldo = ldo;
   hipStream_t s = (hipStream_t)stream;
   if (!g_force_edge.load() && fsw::skinny_forward_ok(p)) return launched(fn, fsw::launch_forward_skinny(dtype, p, s));
+  if (!g_force_edge.load() && fsw::fast_path_ok_forward(p)) return launched(fn, fsw::launch_forward_fast(dtype, p, s));
+  return launched(fn, fsw::launch_forward_generic(dtype, p, s));
+}
+
+int fsw_gating_grad_recompute(const void* x, const void* w_gate, const void* w_up,
+                              const void* grad_out, void* grad_xw_up, void* grad_xw_gate, int64_t T,
+                              int64_t D, int64_t I, int64_t ldx, int64_t ldw, int64_t ldo, int dtype,
+                              void* stream) {
+  const char* fn = "fsw_gating_grad_recompute";
+  if (!x || !w_gate || !w_up || !grad_out || !grad_xw_up || !grad_xw_gate)
+    return fail(FSW_ERR_NULL_POINTER, "%s: all six arrays must be non-null", fn);
+  if (!dtype_ok(dtype)) return fail(FSW_ERR_BAD_DTYPE, "%s: dtype %d is neither bf16 (0) nor fp16 (1)", fn, dtype);
+  if (int e = check_dims(fn, T, D, I)) return e;
+  if (int e = check_ld(fn, "ldx", ldx, D)) return e;
+  if (int e = check_ld(fn, "ldw", ldw, I)) return e;
+  if (int e = check_ld(fn, "ldo", ldo, I)) return e;
+  if (!al2(x) || !al2(w_gate) || !al2(w_up) || !al2(grad_out) || !al2(grad_xw_up) || !al2(grad_xw_gate))
+    return fail(FSW_ERR_ALIGNMENT, "%s: pointers must be 2-byte aligned", fn);
+  fsw::Problem p{};
+  p.x = x; p.wg = w_gate; p.wu = w_up; p.dout = grad_out; p.g = grad_xw_gate; p.u = grad_xw_up;
+  p.T = T; p.D = D; p.I = I; p.ldx = ldx; p.ldw = ldw; p.ldo = ldo;
+  hipStream_t s = (hipStream_t)stream;
   if (!g_force_edge.load() && fsw::fast_path_ok_forward(p)) return launched(fn, fsw::launch_forward_fast(dtype, p, s));
   return launched(fn, fsw::launch_forward_generic(dtype, p, s));
 }

@@ -61,6 +61,13 @@ struct FP16 {
 // silu(g) * u and the gating gradients, fp32 throughout, one rounding at the store.
 FSW_DEV float sigmoidf_fast(float z) { return __frcp_rn(1.0f + __expf(-z)); }
 FSW_DEV float silu_mul(float g, float u) { return g * sigmoidf_fast(g) * u; }
+// dU = dout * silu(g), dG = dout * u * silu'(g), silu'(z) = s + z*s*(1 - s), s = sigmoid(z)
+FSW_DEV void gating_grad(float dout, float g, float u, float& dU, float& dG) {
+  const float s = sigmoidf_fast(g);
+  const float zs = g * s;
+  dU = dout * zs;
+  dG = dout * u * (s + zs * (1.0f - s));
+}
 
 // ---- raw buffer descriptors and direct-to-LDS loads -------------------------
 // Word 3 for gfx90a/gfx94x/gfx950 raw buffers (32-bit data format, no swizzle).

@@ -11,11 +11,10 @@ namespace fsw {
 template <typename E>
 FSW_DEV void gate_grad(unsigned short dout, unsigned short g, unsigned short u, unsigned short& dU,
                        unsigned short& dG) {
-  const float d = E::to_float(dout), z = E::to_float(g), uu = E::to_float(u);
-  const float s = sigmoidf_fast(z);
-  const float zs = z * s;
-  dU = E::from_float(d * zs);
-  dG = E::from_float(d * uu * (s + zs * (1.0f - s)));
+  float fu, fg;
+  gating_grad(E::to_float(dout), E::to_float(g), E::to_float(u), fu, fg);
+  dU = E::from_float(fu);
+  dG = E::from_float(fg);
 }
 
 template <typename E>

@@ -27,6 +27,9 @@ struct GemmParams {
   void* c0;        // kFwd: out    kDx: dx     kDw: dWg
   void* c1;        // kFwd: g (may be null)    kDw: dWu
   void* c2;        // kFwd: u (may be null)
+  // kFwd only, gating-gradient mode (d0 != null): nothing is written to c0; c1 = dG, c2 = dU with
+  // dU = d0 * silu(g), dG = d0 * u * silu'(g) computed from the fp32 accumulators (d0 has ldc too)
+  const void* d0;
   int M, N, K;     // GEMM view: kFwd (T,I,D)  kDx (T,D,I)  kDw (D,I,T)
   int lda, ldb, ldc;  // leading dimensions in elements
   int tiles_m, tiles_n, group_m;
@@ -350,9 +353,25 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
 #pragma unroll
   for (int q = 0; q < 2; q++) {  // 32 rows of the wave's 64 at a time
     if constexpr (MODE == kFwd) {
-      // out = silu(g) * u, then g and u themselves (skipped when the caller passes no buffers for them)
+      // gating-gradient mode: this lane's upstream gradients, 4 consecutive columns per 16x16 block
+      u32x2 dv[2][4];
+      const bool gating = p.d0 != nullptr;
+      if (gating) {
+#pragma unroll
+        for (int mbl = 0; mbl < 2; mbl++)
+#pragma unroll
+          for (int c = 0; c < 4; c++) {
+            const int m = m0 + wm * 64 + (2 * q + mbl) * 16 + (lane & 15);
+            const int n = n0 + wn * 64 + c * 16 + 4 * (lane >> 4);
+            dv[mbl][c] = (m < p.M && n < p.N) ? *(const u32x2*)((const unsigned short*)p.d0 + (size_t)m * p.ldc + n)
+                                              : u32x2{0u, 0u};
+          }
+      }
+      // out = silu(g) * u, then g and u themselves (skipped when the caller passes no buffers for them);
+      // in gating-gradient mode dG and dU take the places of g and u and out is not written
 #pragma unroll
       for (int which = 0; which < 3; which++) {
+        if (which == 0 && gating) continue;
         if (which > 0 && p.c1 == nullptr) break;
 #pragma unroll
         for (int mbl = 0; mbl < 2; mbl++)
@@ -361,7 +380,16 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
             const f32x4 g = acc[c][2 * q + mbl], u = acc[4 + c][2 * q + mbl];
             float v[4];
 #pragma unroll
-            for (int e = 0; e < 4; e++) v[e] = which == 0 ? silu_mul(g[e], u[e]) : (which == 1 ? g[e] : u[e]);
+            for (int e = 0; e < 4; e++) {
+              if (gating) {
+                const unsigned w = e < 2 ? dv[mbl][c].x : dv[mbl][c].y;
+                float dU, dG;
+                gating_grad(E::to_float((unsigned short)((e & 1) ? (w >> 16) : (w & 0xffffu))), g[e], u[e], dU, dG);
+                v[e] = which == 1 ? dG : dU;
+              } else {
+                v[e] = which == 0 ? silu_mul(g[e], u[e]) : (which == 1 ? g[e] : u[e]);
+              }
+            }
             *(FSW_LDS u32x2*)(patch + wr_off + mbl * 16 * kPatchPitch + c * 32) = pack4(v[0], v[1], v[2], v[3]);
           }
         unsigned short* dst = (unsigned short*)(which == 0 ? p.c0 : (which == 1 ? p.c1 : p.c2));

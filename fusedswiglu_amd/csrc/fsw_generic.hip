@@ -16,6 +16,8 @@ struct GenericParams {
   int passes;   // 1, or 2 for dx (second pass accumulates into the same tile)
   int dual;     // 1: two B matrices -> two results sharing A;  0: one result
   int swiglu;   // 1: c[0] = silu(acc0)*acc1, c[1] = acc0, c[2] = acc1 (c[1], c[2] may be null)
+                // 2: gating gradients from the recomputed pre-activations: c[1] = dG, c[2] = dU
+  const unsigned short* dout;  // swiglu == 2: upstream gradient, leading dimension ldc
 };
 
 constexpr int kGT = 64;      // tile edge
@@ -81,7 +83,12 @@ __global__ __launch_bounds__(256) void generic_kernel(GenericParams p) {
     const int n = n0 + wn * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
     if (n >= p.N) continue;
     const long long o = (long long)m * p.ldc + n;
-    if (p.swiglu) {
+    if (p.swiglu == 2) {
+      float dU, dG;
+      gating_grad(E::to_float(p.dout[o]), acc[0][r], acc[1][r], dU, dG);
+      p.c[1][o] = E::from_float(dG);
+      p.c[2][o] = E::from_float(dU);
+    } else if (p.swiglu) {
       p.c[0][o] = E::from_float(silu_mul(acc[0][r], acc[1][r]));
       if (p.c[1]) { p.c[1][o] = E::from_float(acc[0][r]); p.c[2][o] = E::from_float(acc[1][r]); }
     } else {
@@ -109,6 +116,7 @@ hipError_t launch_forward_generic(int dtype, const Problem& p, hipStream_t s) {
   g.c[0] = (us)p.out; g.c[1] = (us)p.g; g.c[2] = (us)p.u;
   g.a_sm = p.ldx; g.a_sk = 1; g.b_sk = p.ldw; g.b_sn = 1; g.ldc = p.ldo;
   g.M = (int)p.T; g.N = (int)p.I; g.K = (int)p.D; g.passes = 1; g.dual = 1; g.swiglu = 1;
+  if (p.dout) { g.swiglu = 2; g.dout = (cus)p.dout; }
   return launch_generic(dtype, g, s);
 }
 

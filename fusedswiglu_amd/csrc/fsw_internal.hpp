@@ -12,6 +12,8 @@ struct Problem {
   const void *x, *wg, *wu;       // x [T,D]; Wg, Wu [D,I]
   const void *dG, *dU;           // [T,I]
   void *out, *g, *u;             // [T,I]   (g, u may be null in the forward)
+  const void* dout;              // [T,I]   non-null: the forward recomputes g, u and writes the gating
+                                 //         gradients dG -> g, dU -> u instead (out is not written)
   void *dx;                      // [T,D]
   void *dWg, *dWu;               // [D,I]
   long long T, D, I;

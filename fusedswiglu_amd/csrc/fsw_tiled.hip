@@ -15,7 +15,7 @@ static bool dims_ok(const Problem& p) {
 
 bool fast_path_ok_forward(const Problem& p) {
   return dims_ok(p) && ld_ok(p.ldx) && ld_ok(p.ldw) && mult8(p.ldo) && al16(p.x) && al16(p.wg) &&
-         al16(p.wu) && al16(p.out) && al16(p.g) && al16(p.u);
+         al16(p.wu) && al16(p.out) && al16(p.g) && al16(p.u) && al16(p.dout);
 }
 bool fast_path_ok_input_grad(const Problem& p) {
   return dims_ok(p) && ld_ok(p.ldo) && ld_ok(p.ldw) && mult8(p.lddx) && al16(p.dG) && al16(p.dU) &&
@@ -115,7 +115,7 @@ static hipError_t launch(int dtype, GemmParams g, hipStream_t s, void* ws = null
 
 hipError_t launch_forward_fast(int dtype, const Problem& p, hipStream_t s) {
   GemmParams g{};
-  g.a0 = p.x; g.b0 = p.wg; g.b1 = p.wu; g.c0 = p.out; g.c1 = p.g; g.c2 = p.u;
+  g.a0 = p.x; g.b0 = p.wg; g.b1 = p.wu; g.c0 = p.out; g.c1 = p.g; g.c2 = p.u; g.d0 = p.dout;
   g.M = (int)p.T; g.N = (int)p.I; g.K = (int)p.D;
   g.lda = (int)p.ldx; g.ldb = (int)p.ldw; g.ldc = (int)p.ldo;
   return launch<kFwd>(dtype, g, s);

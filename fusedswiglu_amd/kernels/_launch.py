@@ -116,6 +116,37 @@ def elementwise_backward(grad_output: torch.Tensor, xw_gate: torch.Tensor, xw_up
     return grad_xw_up, grad_xw_gate
 
 
+def gating_grad_recompute(grad_output: torch.Tensor, x: torch.Tensor, w_gate: torch.Tensor,
+                          w_up: torch.Tensor, dtype: torch.dtype) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(grad_xw_up, grad_xw_gate) like elementwise_backward, but from x and the weights: the
+    pre-activations x@w_gate and x@w_up are recomputed in fp32 inside the kernel and never stored.
+    For backward passes that did not save them (fused_swiglu/swiglu.py:28 saves them always)."""
+    _require(x.ndim >= 2 and w_up.ndim == 2 and w_gate.ndim == 2,
+             "Incorrect number of dimensions for LHS or RHS")
+    _require(x.shape[-1] == w_up.shape[0],
+             f"Dimension mismatch. Expected x.shape[-1] ({x.shape[-1]}) to be equal to "
+             f"w_up.shape[0] ({w_up.shape[0]})")
+    _require(w_up.shape == w_gate.shape, "Expected both weight matrices to have same shape")
+    D, I = w_up.shape
+    _require(tuple(grad_output.shape) == tuple(x.shape[:-1]) + (I,),
+             f"grad_output {tuple(grad_output.shape)} does not match x {tuple(x.shape)} and I = {I}")
+    _require(all(t.dtype == dtype for t in (grad_output, x, w_gate, w_up)), f"Expected {dtype} tensors")
+    dev = _check_device(grad_output, x, w_gate, w_up)
+    _require(x.numel() > 0 and I > 0, "empty input")
+    x2, wg, wu = _rows(x), _rows(w_gate), _rows(w_up)
+    if _ld(wg) != _ld(wu):
+        wg, wu = wg.contiguous(), wu.contiguous()
+    dout = grad_output.contiguous()
+    grad_xw_up = torch.empty_like(dout)
+    grad_xw_gate = torch.empty_like(dout)
+    with torch.cuda.device(dev):
+        _abi.check(_abi.lib().fsw_gating_grad_recompute(
+            x2.data_ptr(), wg.data_ptr(), wu.data_ptr(), dout.data_ptr(), grad_xw_up.data_ptr(),
+            grad_xw_gate.data_ptr(), x2.shape[0], D, I, _ld(x2), _ld(wg), I, _DTYPE_CODE[dtype],
+            _stream_ptr(dev)))
+    return grad_xw_up, grad_xw_gate
+
+
 def fused_input_grad(grad_xw_gate: torch.Tensor, grad_xw_up: torch.Tensor, w_gate: torch.Tensor,
                      w_up: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
     """grad_x = grad_xw_gate @ w_gate.T + grad_xw_up @ w_up.T in one kernel (swiglu.py:45)."""

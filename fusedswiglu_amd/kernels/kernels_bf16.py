@@ -10,6 +10,7 @@ ShapeError = _launch.ShapeError
 
 fused_swiglu_fwd = partial(_launch.fused_swiglu_fwd, dtype=_DT)
 elementwise_backward = partial(_launch.elementwise_backward, dtype=_DT)
+gating_grad_recompute = partial(_launch.gating_grad_recompute, dtype=_DT)
 fused_input_grad = partial(_launch.fused_input_grad, dtype=_DT)
 fused_weight_grad = partial(_launch.fused_weight_grad, dtype=_DT)
 fused_bmm = partial(_launch.fused_bmm, dtype=_DT)

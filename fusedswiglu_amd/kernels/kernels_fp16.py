@@ -20,6 +20,7 @@ def fused_swiglu_fwd(x, w_gate, w_up, fast_accum: bool = True, save_preactivatio
 
 
 elementwise_backward = partial(_launch.elementwise_backward, dtype=_DT)
+gating_grad_recompute = partial(_launch.gating_grad_recompute, dtype=_DT)
 fused_input_grad = partial(_launch.fused_input_grad, dtype=_DT)
 fused_weight_grad = partial(_launch.fused_weight_grad, dtype=_DT)
 fused_bmm = partial(_launch.fused_bmm, dtype=_DT)

@@ -4,7 +4,9 @@ The reference stops at `FusedSwiGLU.apply(x, w_gate, w_up)` and leaves holding t
 user (README.md:25-38).  `SwiGLU` owns them in the layout the kernels want ([d_model,
 d_intermediate], unit inner stride), initialised like the reference's tests draw them
 (N(0, 1)/sqrt(d_model), test_swiglu.py:30-35), either as two parameters or as one packed
-[d_model, 2*d_intermediate] parameter [w_gate | w_up]."""
+[d_model, 2*d_intermediate] parameter [w_gate | w_up].  `recompute=True` keeps no pre-activations
+between forward and backward (2*T*d_intermediate elements less per call) and recomputes them in the
+backward's gating-gradient kernel."""
 from __future__ import annotations
 
 import torch
@@ -15,11 +17,12 @@ from . import ops
 
 class SwiGLU(nn.Module):
     def __init__(self, d_model: int, d_intermediate: int, dtype: torch.dtype = torch.bfloat16,
-                 device=None, packed: bool = False):
+                 device=None, packed: bool = False, recompute: bool = False):
         super().__init__()
         if dtype not in (torch.bfloat16, torch.float16):
             raise ValueError(f"SwiGLU computes in bfloat16 or float16, got {dtype}")
         self.d_model, self.d_intermediate, self.packed = d_model, d_intermediate, packed
+        self.recompute = recompute
         kw = dict(device=device, dtype=dtype)
         if packed:
             self.w_gate_up = nn.Parameter(torch.empty(d_model, 2 * d_intermediate, **kw))
@@ -37,8 +40,8 @@ class SwiGLU(nn.Module):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         dtype = next(self.parameters()).dtype
         if self.packed:
-            return ops.swiglu_packed(x, self.w_gate_up, autocast_dtype=dtype)
-        return ops.swiglu(x, self.w_gate, self.w_up, autocast_dtype=dtype)
+            return ops.swiglu_packed(x, self.w_gate_up, autocast_dtype=dtype, recompute=self.recompute)
+        return ops.swiglu(x, self.w_gate, self.w_up, autocast_dtype=dtype, recompute=self.recompute)
 
     def extra_repr(self) -> str:
-        return f"d_model={self.d_model}, d_intermediate={self.d_intermediate}, packed={self.packed}"
+        return f"d_model={self.d_model}, d_intermediate={self.d_intermediate}, packed={self.packed}, recompute={self.recompute}"

@@ -9,7 +9,10 @@ that a traced program keeps them as opaque calls into libfusedswiglu:
     fusedswiglu_amd::swiglu_backward(grad_out, x, w_gate, w_up, xw_gate, xw_up,
                                      need_x, need_w_gate, need_w_up, packed) -> (dx, dw_gate, dw_up)
 
-`swiglu(x, w_gate, w_up)` and `swiglu_packed(x, w_gate_up)` are the functional entry points.  The
+`swiglu(x, w_gate, w_up)` and `swiglu_packed(x, w_gate_up)` are the functional entry points.  With
+`recompute=True` the forward keeps only x and the weights for the backward (fused_swiglu/swiglu.py:28
+also keeps x@w_gate and x@w_up, 2*T*I elements); the backward then recomputes both products inside
+the gating-gradient kernel, trading 4*T*D*I flops for that memory.  The
 element type (bfloat16 or float16) is taken from the tensors; under CUDA autocast the arguments are
 cast to `autocast_dtype` first, as `custom_fwd(cast_inputs=...)` does for the reference's Functions
 (swiglu.py:18, swiglu_f16.py:18).  Gradient order follows swiglu.py:58: (dx, dw_gate, dw_up).
@@ -69,11 +72,15 @@ def swiglu_backward(grad_out: Tensor, x: Tensor, w_gate: Tensor, w_up: Tensor, x
     """(dx, dw_gate, dw_up); a gradient that is not needed comes back with zero elements.  With
     `packed`, the second result is ONE [D, 2I] array [dw_gate | dw_up] written in place by the
     weight-gradient kernel (row stride 2I) and the third is empty: the gradient of a packed weight
-    without a concatenation."""
+    without a concatenation.  Empty xw_gate / xw_up (a forward that did not save them) switch to the
+    recomputing gating-gradient kernel."""
     dtype = _dtype_of(x)
     if grad_out.dtype != dtype:
         grad_out = grad_out.to(dtype)
-    d_up, d_gate = _launch.elementwise_backward(grad_out, xw_gate, xw_up, dtype)
+    if xw_gate.numel() == 0:
+        d_up, d_gate = _launch.gating_grad_recompute(grad_out, x, w_gate, w_up, dtype)
+    else:
+        d_up, d_gate = _launch.elementwise_backward(grad_out, xw_gate, xw_up, dtype)
     dx = dw_gate = dw_up = None
     if need_x:
         dx = _launch.fused_input_grad(d_gate, d_up, w_gate, w_up, dtype)
@@ -128,13 +135,14 @@ def _autocast(dtype, *tensors):
     return tensors
 
 
-def swiglu(x: Tensor, w_gate: Tensor, w_up: Tensor, autocast_dtype: torch.dtype | None = torch.bfloat16) -> Tensor:
+def swiglu(x: Tensor, w_gate: Tensor, w_up: Tensor, autocast_dtype: torch.dtype | None = torch.bfloat16,
+           recompute: bool = False) -> Tensor:
     """silu(x @ w_gate) * (x @ w_up) with weights laid out [d_model, d_intermediate]."""
     _require_gpu(x, w_gate, w_up)
     x, w_gate, w_up = _autocast(autocast_dtype, x, w_gate, w_up)
     with torch.autocast(device_type="cuda", enabled=False):
         save = torch.is_grad_enabled() and (x.requires_grad or w_gate.requires_grad or w_up.requires_grad)
-        return swiglu_forward(x, w_gate, w_up, save)[0]
+        return swiglu_forward(x, w_gate, w_up, save and not recompute)[0]
 
 
 class _PackedSwiGLU(torch.autograd.Function):
@@ -143,10 +151,10 @@ class _PackedSwiGLU(torch.autograd.Function):
     array, so packing costs no copies in either direction."""
 
     @staticmethod
-    def forward(ctx, x, w_gate_up):
+    def forward(ctx, x, w_gate_up, recompute):
         I = w_gate_up.shape[1] // 2
         w_gate, w_up = w_gate_up[:, :I], w_gate_up[:, I:]
-        out, g, u = swiglu_forward(x, w_gate, w_up, True)
+        out, g, u = swiglu_forward(x, w_gate, w_up, not recompute)
         ctx.save_for_backward(x, w_gate_up, g, u)
         return out
 
@@ -154,13 +162,14 @@ class _PackedSwiGLU(torch.autograd.Function):
     def backward(ctx, grad_out):
         x, w_gate_up, g, u = ctx.saved_tensors
         I = w_gate_up.shape[1] // 2
-        need_x, need_w = ctx.needs_input_grad
+        need_x, need_w = ctx.needs_input_grad[:2]
         dx, dw, _ = swiglu_backward(grad_out.contiguous(), x, w_gate_up[:, :I], w_gate_up[:, I:], g, u,
                                     need_x, need_w, need_w, True)
-        return (dx if need_x else None), (dw if need_w else None)
+        return (dx if need_x else None), (dw if need_w else None), None
 
 
-def swiglu_packed(x: Tensor, w_gate_up: Tensor, autocast_dtype: torch.dtype | None = torch.bfloat16) -> Tensor:
+def swiglu_packed(x: Tensor, w_gate_up: Tensor, autocast_dtype: torch.dtype | None = torch.bfloat16,
+                  recompute: bool = False) -> Tensor:
     """SwiGLU with a packed weight [d_model, 2*d_intermediate] = [w_gate | w_up]."""
     if w_gate_up.ndim != 2 or w_gate_up.shape[1] % 2:
         raise _launch.ShapeError("packed weight must be [d_model, 2*d_intermediate]")
@@ -168,6 +177,6 @@ def swiglu_packed(x: Tensor, w_gate_up: Tensor, autocast_dtype: torch.dtype | No
     x, w_gate_up = _autocast(autocast_dtype, x, w_gate_up)
     with torch.autocast(device_type="cuda", enabled=False):
         if torch.is_grad_enabled() and (x.requires_grad or w_gate_up.requires_grad):
-            return _PackedSwiGLU.apply(x, w_gate_up)
+            return _PackedSwiGLU.apply(x, w_gate_up, recompute)
         I = w_gate_up.shape[1] // 2
         return swiglu_forward(x, w_gate_up[:, :I], w_gate_up[:, I:], False)[0]

@@ -56,7 +56,8 @@ const char* fsw_status_string(int status);
 /* Message of the calling thread's most recent failed call ("" if none). */
 const char* fsw_last_error(void);
 /* 1 if the arguments of the named step would run on the tiled kernels, 0 if on the
- * edge-shape kernel.  step: 0 forward, 1 input_grad, 2 weight_grad.  Pure host logic. */
+ * edge-shape kernel.  step: 0 forward, 1 input_grad, 2 weight_grad, 3 gating_grad_recompute.
+ * Pure host logic. */
 int fsw_uses_tiled_kernel(int step, int64_t T, int64_t D, int64_t I, int64_t ldx, int64_t ldw,
                           int64_t ldo, int64_t ld_grad, unsigned pointer_alignment);
 /* Test hook: nonzero forces every later call of this process onto the edge-shape kernels. */
@@ -83,6 +84,19 @@ int fsw_swiglu_forward(const void* x, const void* w_gate, const void* w_up, void
 int fsw_elementwise_backward(const void* grad_out, const void* xw_gate, const void* xw_up,
                              void* grad_xw_up, void* grad_xw_gate, int64_t numel, int dtype,
                              void* stream);
+
+/*
+ * Gating gradient without saved pre-activations: recomputes g = x Wg and u = x Wu (fp32, never
+ * stored) and writes grad_xw_up = grad_out * silu(g), grad_xw_gate = grad_out * u * silu'(g).
+ * Stands in for the pair "save x@Wg, x@Wu in the forward (fused_swiglu/swiglu.py:28) + elementwise_backward
+ * (kernels_bf16.py:236-255)" for callers that prefer 4*T*D*I extra flops to keeping 2*T*I saved
+ * elements per layer; the reference has no such mode.
+ *   x [T,D] (ldx)   w_gate, w_up [D,I] (ldw)   grad_out, grad_xw_up, grad_xw_gate [T,I] (ldo)
+ */
+int fsw_gating_grad_recompute(const void* x, const void* w_gate, const void* w_up,
+                              const void* grad_out, void* grad_xw_up, void* grad_xw_gate, int64_t T,
+                              int64_t D, int64_t I, int64_t ldx, int64_t ldw, int64_t ldo, int dtype,
+                              void* stream);
 
 /*
  * Optional scratch for the two gradient GEMMs.  When a problem has too few output tiles to fill the

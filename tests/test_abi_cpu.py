@@ -63,6 +63,12 @@ def test_backward_validation(L):
     assert e(P, P, None, P, P, 8, 0, None) == 1
     assert e(P, P, P, P, P, 0, 0, None) == 3
     assert e(P, P, P, P, P, 8, 2, None) == 2
+    rc = L.fsw_gating_grad_recompute
+    assert rc(P, P, P, None, P, P, 8, 8, 8, 8, 8, 8, 0, None) == 1
+    assert rc(P, P, P, P, P, P, 8, 8, 8, 8, 8, 8, 5, None) == 2
+    assert rc(P, P, P, P, P, P, 8, 0, 8, 8, 8, 8, 0, None) == 3
+    assert rc(P, P, P, P, P, P, 8, 8, 16, 8, 16, 8, 0, None) == 4  # ldo < I
+    assert rc(P, P, P, ctypes.c_void_p(0x1001), P, P, 8, 8, 8, 8, 8, 8, 0, None) == 5
     dx = L.fsw_input_grad
     assert dx(P, P, P, P, None, 8, 8, 8, 8, 8, 8, None, 0, 0, None) == 1
     assert dx(P, P, P, P, P, 8, 8, 8, 8, 8, 4, None, 0, 0, None) == 4  # ld_dx < D
@@ -82,9 +88,10 @@ def test_backward_validation(L):
 def test_kernel_selection_logic(L):
     t = L.fsw_uses_tiled_kernel
     # the north-star shape and the fp16 config run on the tiled kernels in all three steps
-    for step in range(3):
+    for step in range(4):
         assert t(step, 8192, 4096, 12288, 4096, 12288, 12288, 4096 if step == 1 else 12288, 16) == 1
         assert t(step, 8192, 4096, 11008, 4096, 11008, 11008, 4096 if step == 1 else 11008, 16) == 1
+    assert t(3, 8192, 4096, 11007, 4096, 11007, 11007, 11007, 16) == 0 and t(4, 8, 8, 8, 8, 8, 8, 8, 16) == 0
     # dimensions that are not multiples of 8, or unaligned pointers, take the edge-shape kernel
     assert t(0, 8192, 4096, 11007, 4096, 11007, 11007, 11007, 16) == 0
     assert t(0, 8192, 4100, 12288, 4100, 12288, 12288, 12288, 16) == 0

@@ -145,3 +145,56 @@ def test_torch_compile_keeps_the_operator_opaque(oracle):
     torch.cuda.synchronize()
     assert torch.equal(oc, oe)
     assert torch.equal(xc.grad, ge[0]) and torch.equal(m.w_gate.grad, ge[1]) and torch.equal(m.w_up.grad, ge[2])
+
+
+# ---- backward without saved pre-activations -----------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("shape", [(2, 136, 264, 520), (1, 300, 256, 384), (3, 50, 72, 65), (1, 7, 8, 8), (1, 257, 100, 130)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_gating_grad_recompute_launcher(oracle, dtype, shape):
+    """fsw_gating_grad_recompute against the oracle's gating gradient evaluated on the exact
+    pre-activations (tiled kernel for 8-aligned shapes, edge-shape kernel otherwise)."""
+    from fusedswiglu_amd.kernels import kernels_bf16, kernels_fp16
+    k = kernels_bf16 if dtype == torch.bfloat16 else kernels_fp16
+    (x, wg, wu, dy), (tx, twg, twu, tdy) = inputs(oracle, shape, dtype, seed=21)
+    dU, dG = k.gating_grad_recompute(tdy, tx, twg, twu)
+    torch.cuda.synchronize()
+    _, g, u = oracle.fused_swiglu_fwd(x, wg, wu)
+    o_dU, o_dG = oracle.elementwise_backward(dy, g, u)
+    assert dU.shape == tdy.shape and dG.shape == tdy.shape
+    assert oracle.rel_error(np64(dU), o_dU) < TOL[dtype] and oracle.rel_error(np64(dG), o_dG) < TOL[dtype]
+    assert oracle.rel_error(np64(dU), o_dG) > 0.1  # (up, gate) order as in elementwise_backward
+
+
+@pytest.mark.parametrize("packed", [False, True], ids=["two_weights", "packed"])
+def test_recompute_backward_saves_no_preactivations(oracle, packed):
+    dtype, shape = torch.bfloat16, (2, 136, 264, 520)
+    (x, wg, wu, dy), (tx, twg, twu, tdy) = inputs(oracle, shape, dtype, seed=22)
+    T, I = shape[0] * shape[1], shape[3]
+    grads, saved_elems = {}, {}
+    for recompute in (False, True):
+        m = fsw.SwiGLU(shape[2], shape[3], dtype=dtype, device=DEV, packed=packed, recompute=recompute)
+        with torch.no_grad():
+            if packed:
+                m.w_gate_up.copy_(torch.cat([twg, twu], dim=1))
+            else:
+                m.w_gate.copy_(twg)
+                m.w_up.copy_(twu)
+        xin = tx.clone().requires_grad_(True)
+        sizes = []
+        with torch.autograd.graph.saved_tensors_hooks(lambda t: (sizes.append(t.numel()), t)[1], lambda t: t):
+            out = m(xin)
+        out.backward(tdy)
+        torch.cuda.synchronize()
+        saved_elems[recompute] = sum(sizes)
+        w = m.w_gate_up.grad if packed else torch.cat([m.w_gate.grad, m.w_up.grad], dim=1)
+        grads[recompute] = (out.detach(), xin.grad, w)
+    assert saved_elems[False] - saved_elems[True] == 2 * T * I
+    o_out = oracle.fused_swiglu_fwd(x, wg, wu)[0]
+    o_dx, o_dwg, o_dwu = oracle.swiglu_backward(x, wg, wu, dy)
+    out, dx, dw = grads[True]
+    assert torch.equal(out, grads[False][0])
+    assert oracle.rel_error(np64(out), o_out) < 1e-2 and oracle.rel_error(np64(dx), o_dx) < 1e-2
+    assert oracle.rel_error(np64(dw[:, :I]), o_dwg) < 1e-2 and oracle.rel_error(np64(dw[:, I:]), o_dwu) < 1e-2
+    # recomputed pre-activations are not rounded to 16 bits first: not worse than the saving path
+    assert oracle.rel_error(np64(dx), o_dx) <= 1.05 * oracle.rel_error(np64(grads[False][1]), o_dx)
