@@ -27,9 +27,9 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # (FETCH_SIZE scaled by 2.0, WRITE_SIZE by 1.0 against a plain 1 GiB copy).  bench.py cannot run the
 # profiler itself; this table is refreshed whenever that profile is.
 PROFILED_TRAFFIC_BYTES = {
-    "forward_dual_gemm": (2 * 1179903 + 589824) * 1024,
-    "input_grad_dual_gemm": (2 * 1183105 + 65536) * 1024,
-    "weight_grad_dual_gemm": (2 * 1473863 + 196608) * 1024,
+    "forward_dual_gemm": (2 * 1180115 + 589824) * 1024,
+    "input_grad_dual_gemm": (2 * 1180438 + 65536) * 1024,
+    "weight_grad_dual_gemm": (2 * 1179789 + 196608) * 1024,
 }
 
 
