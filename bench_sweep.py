@@ -16,18 +16,24 @@ import os
 sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 
 
-def time_ms(fn, iters, warmup=3):
+def time_ms(fn, iters, warmup=3, min_ms=40.0):
+    """Mean time per call: `iters` calls, repeated until the timed region is at least `min_ms` long
+    (the small shapes of the sweep run a few microseconds per call)."""
     import torch
 
     for _ in range(warmup):
         fn()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(iters):
-        fn()
-    e1.record()
-    e1.synchronize()
-    return e0.elapsed_time(e1) / iters
+    while True:
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+        e1.synchronize()
+        total = e0.elapsed_time(e1)
+        if total >= min_ms or iters >= 100000:
+            return total / iters
+        iters = int(iters * max(2.0, 1.2 * min_ms / max(total, 1e-3)))
 
 
 def main():
