@@ -37,6 +37,42 @@ class SwiGLU(nn.Module):
             if p.device.type != "meta":
                 nn.init.normal_(p, mean=0.0, std=std)
 
+    @classmethod
+    def from_linear(cls, gate_proj: nn.Linear, up_proj: nn.Linear, dtype: torch.dtype = None,
+                    packed: bool = False, recompute: bool = False) -> "SwiGLU":
+        """Build from the usual pair of bias-free `nn.Linear(d_model, d_intermediate)` projections,
+        whose weights are stored [d_intermediate, d_model]: they are transposed once into the
+        [d_model, d_intermediate] layout this path computes on."""
+        if gate_proj.bias is not None or up_proj.bias is not None:
+            raise ValueError("SwiGLU has no bias terms")
+        if gate_proj.weight.shape != up_proj.weight.shape:
+            raise ValueError("gate and up projections must have the same shape")
+        d_int, d_model = gate_proj.weight.shape
+        dtype = dtype or gate_proj.weight.dtype
+        m = cls(d_model, d_int, dtype=dtype, device=gate_proj.weight.device, packed=packed, recompute=recompute)
+        with torch.no_grad():
+            wg, wu = gate_proj.weight.t().to(dtype), up_proj.weight.t().to(dtype)
+            if packed:
+                m.w_gate_up.copy_(torch.cat([wg, wu], dim=1))
+            else:
+                m.w_gate.copy_(wg)
+                m.w_up.copy_(wu)
+        return m
+
+    def to_linear(self):
+        """The inverse of from_linear: (gate_proj, up_proj) as bias-free nn.Linear modules."""
+        if self.packed:
+            wg, wu = self.w_gate_up[:, :self.d_intermediate], self.w_gate_up[:, self.d_intermediate:]
+        else:
+            wg, wu = self.w_gate, self.w_up
+        out = []
+        for w in (wg, wu):
+            lin = nn.Linear(self.d_model, self.d_intermediate, bias=False, device=w.device, dtype=w.dtype)
+            with torch.no_grad():
+                lin.weight.copy_(w.t())
+            out.append(lin)
+        return tuple(out)
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         dtype = next(self.parameters()).dtype
         if self.packed:

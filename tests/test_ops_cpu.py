@@ -43,3 +43,18 @@ def test_host_tensors_and_bad_shapes_are_rejected_before_any_launch():
         m(torch.zeros(2, 16, dtype=torch.bfloat16))
     with pytest.raises(kernels_bf16.ShapeError, match="packed weight"):
         fsw.swiglu_packed(torch.zeros(2, 16), torch.zeros(16, 25))
+
+
+def test_module_from_and_to_linear():
+    gate = torch.nn.Linear(32, 48, bias=False, dtype=torch.bfloat16)
+    up = torch.nn.Linear(32, 48, bias=False, dtype=torch.bfloat16)
+    for packed in (False, True):
+        m = fsw.SwiGLU.from_linear(gate, up, packed=packed)
+        assert (m.d_model, m.d_intermediate) == (32, 48)
+        wg = m.w_gate_up[:, :48] if packed else m.w_gate
+        wu = m.w_gate_up[:, 48:] if packed else m.w_up
+        assert torch.equal(wg, gate.weight.t()) and torch.equal(wu, up.weight.t())
+        g2, u2 = m.to_linear()
+        assert torch.equal(g2.weight, gate.weight) and torch.equal(u2.weight, up.weight)
+    with pytest.raises(ValueError):
+        fsw.SwiGLU.from_linear(torch.nn.Linear(8, 8), up)
