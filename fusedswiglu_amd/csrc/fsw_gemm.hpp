@@ -46,17 +46,13 @@ constexpr int kMcSlots = 4;
 constexpr int kMcSlotBytes = 2 * kMcPanelBytes;  // two 128-column panels: 16 KiB
 constexpr int kKcAreaBytes = 256 * 128;          // 256 rows x 64 k-elements: 32 KiB
 
-#ifndef FSW_KC_AREAS_A
-#define FSW_KC_AREAS_A 3
-#endif
-
 template <int MODE>
 struct Cfg {
   static constexpr bool kAKc = (MODE != kDw);
   static constexpr bool kBKc = (MODE == kDx);
   static constexpr int kTileN = (MODE == kDx) ? 256 : 128;
   // KC rings: number of 32 KiB areas.  160 KiB of LDS in all for kFwd and kDx, 128 KiB for kDw.
-  static constexpr int kAreasA = FSW_KC_AREAS_A;
+  static constexpr int kAreasA = 3;
   static constexpr int kAreasB = 2;
   static constexpr int kBytesA = kAKc ? kAreasA * kKcAreaBytes : kMcSlots * kMcSlotBytes;
   static constexpr int kBytesB = kBKc ? kAreasB * kKcAreaBytes : kMcSlots * kMcSlotBytes;
@@ -227,25 +223,18 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
     if constexpr (!B_KC) issue_mc(mb, i + C::kAheadB, smem_b);
   };
   // Wait until this wave's share of step kt+1 has landed, then meet the other waves.  Loads complete in
-  // issue order, so it is enough to bound how many of the younger ones may still be in flight.  With
-  // three KC areas for A:
+  // issue order, so it is enough to bound how many of the younger ones may still be in flight:
   //   kFwd  after the MC slot of step kt+1 (issued during step kt-2) come one KC batch (4) and two MC
   //         batches (2+2)                                                                    -> 8
   //   kDw   two steps of 2+2                                                                 -> 8
   //   kDx   step kt odd: after the B pair of kt+1 (issued first during step kt-1) comes only the A pair
   //         issued with it -> 4;  kt even: nothing new is needed, this step's 8 loads are younger -> 12
-  // With two KC areas for A the A pair of step kt+1 is issued during step kt-1 as well:
-  //   kFwd  kt odd: after that A pair come MC(kt+2), MC(kt+3) -> 4;  kt even: as above -> 8
-  //   kDx   kt odd: the A pair is the youngest load -> 0;  kt even: this step's 8 loads -> 8
   // Near the end of the reduction, where some of those loads no longer exist, wait for everything.
   auto wait_next_step_and_barrier = [&](int kt) {
     if (kt + C::kAheadMax >= kt_total) { wait_vmcnt_and_barrier<0>(); return; }
     if constexpr (MODE == kDx) {
-      if (kt & 1) wait_vmcnt_and_barrier<(C::kAreasA == 3 ? 4 : 0)>();
-      else wait_vmcnt_and_barrier<(C::kAreasA == 3 ? 12 : 8)>();
-    } else if constexpr (MODE == kFwd && C::kAreasA == 2) {
       if (kt & 1) wait_vmcnt_and_barrier<4>();
-      else wait_vmcnt_and_barrier<8>();
+      else wait_vmcnt_and_barrier<12>();
     } else {
       wait_vmcnt_and_barrier<8>();
     }
