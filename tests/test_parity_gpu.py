@@ -85,6 +85,35 @@ def test_forward_backward_parity_small(oracle, dtype, shape):
     assert oracle.rel_error(np64(dwg), o_dwu) > 0.1
 
 
+def _random_shapes(n, seed):
+    """Seeded mix of shapes: 8-aligned ones (tiled kernels, ragged tile edges, split reductions,
+    the weight-streaming forward for few tokens) and unaligned ones (edge-shape kernels)."""
+    rng = np.random.default_rng(seed)
+    shapes = []
+    for i in range(n):
+        B = int(rng.integers(1, 4))
+        S = int(rng.choice([1, 3, 17, 64, 100, 255, 256, 300, 513]))
+        if i % 3 == 2:
+            D, I = int(rng.integers(1, 300)), int(rng.integers(1, 400))
+        else:
+            D, I = 8 * int(rng.integers(1, 140)), 8 * int(rng.integers(1, 140))
+        shapes.append((B, S, D, I))
+    return shapes
+
+
+@pytest.mark.parametrize("shape", _random_shapes(24, seed=2024), ids=lambda s: "x".join(map(str, s)))
+def test_forward_backward_parity_random_shapes(oracle, shape):
+    dtype = torch.bfloat16 if (shape[1] + shape[3]) % 2 == 0 else torch.float16
+    (x, wg, wu, dy), (tx, twg, twu, tdy) = make(oracle, shape, dtype, seed=shape[2])
+    out, dx, dwg, dwu = run_fwd_bwd(dtype, tx, twg, twu, tdy)
+    o_out, _, _ = oracle.fused_swiglu_fwd(x, wg, wu)
+    o_dx, o_dwg, o_dwu = oracle.swiglu_backward(x, wg, wu, dy)
+    tol = TOL[dtype]
+    for got, want in ((out, o_out), (dx, o_dx), (dwg, o_dwg), (dwu, o_dwu)):
+        assert torch.isfinite(got).all()
+        assert oracle.rel_error(np64(got), want) < tol
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 def test_launchers_match_oracle_and_reference_orders(oracle, dtype):
     """Each launcher on its own, including the saved pre-activations and the (up, gate) return
