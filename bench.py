@@ -194,7 +194,7 @@ def main():
         w_sets = [((torch.randn(D4, I4, device=dev, dtype=dt) / D4 ** 0.5), (torch.randn(D4, I4, device=dev, dtype=dt) / D4 ** 0.5))
                   for _ in range(2)]
         skinny = []
-        for M in (16, 64, 256):
+        for M in (16, 64, 128, 256):
             xs = torch.randn(M, D4, device=dev, dtype=dt)
             os_ = torch.empty(M, I4, device=dev, dtype=dt)
             state = {"i": 0}
