@@ -295,6 +295,28 @@ def test_large_config_slices(oracle):
     _slice_check(oracle, dtype, tx, twg, twu, tdy, out, dx, dwg, dwu, n_rows=2, n_cols=2)
 
 
+@pytest.mark.parametrize("shape", [(1, 100000, 512, 1536),    # very many tokens: 391 tile rows, long dW reduction
+                                   (1, 520, 32768, 256),      # very deep forward reduction, split dx/dW
+                                   (1, 16, 2097144, 8),       # leading dimension just under the 2^21 limit of the tiled kernels
+                                   (1, 40, 8, 131072),        # one reduction step, very wide
+                                   (1, 70000, 8, 8)],         # tiny matrices, many tokens
+                         ids=lambda s: "x".join(map(str, s)))
+def test_extreme_aspect_ratios(oracle, shape):
+    """Shapes at the corners of what the tiled kernels accept, checked on slices."""
+    dtype = torch.bfloat16
+    B, S, D, I = shape
+    g = torch.Generator(device=DEV).manual_seed(S)
+    tx = torch.randn(B, S, D, device=DEV, dtype=torch.float32, generator=g).to(dtype)
+    twg = (torch.randn(D, I, device=DEV, dtype=torch.float32, generator=g) / D ** 0.5).to(dtype)
+    twu = (torch.randn(D, I, device=DEV, dtype=torch.float32, generator=g) / D ** 0.5).to(dtype)
+    tdy = torch.randn(B, S, I, device=DEV, dtype=torch.float32, generator=g).to(dtype)
+    assert _abi.lib().fsw_uses_tiled_kernel(0, B * S, D, I, D, I, I, I, 16) == 1
+    out, dx, dwg, dwu = run_fwd_bwd(dtype, tx, twg, twu, tdy)
+    for t in (out, dx, dwg, dwu):
+        assert torch.isfinite(t).all()
+    _slice_check(oracle, dtype, tx, twg, twu, tdy, out, dx, dwg, dwu, n_rows=3, n_cols=3)
+
+
 # ---- boundary behaviour ---------------------------------------------------------------------------
 def test_edge_kernels_agree_with_tiled_kernels(oracle):
     """Force the edge-shape kernels onto an aligned problem: both paths meet the oracle."""
