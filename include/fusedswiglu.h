@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define FSW_VERSION 100 /* major*10000 + minor*100 + patch */
+#define FSW_VERSION 200 /* major*10000 + minor*100 + patch */
 
 enum { FSW_DTYPE_BF16 = 0, FSW_DTYPE_FP16 = 1 };
 
