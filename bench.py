@@ -173,6 +173,14 @@ def main():
             run = lambda: _abi.check(L.fsw_probe_mfma(rnd, 20000, ncu, p(sink), stream, ctypes.byref(fl)))  # noqa: E731
             ms = gpu_time_ms(run, iters=3, warmup=1)
             ceil[name] = round(fl.value / ms / 1e9, 1)
+        # the matrix cores beside the tiled kernels' own data movement (reads from LDS, L2-hit loads into LDS)
+        window = torch.empty(8 << 20, device=dev, dtype=torch.uint8).fill_(60)
+        for name, mix in (("mfma_16x16x32_normal_operands_tflops", 0), ("mfma_with_kernel_data_movement_tflops", 1)):
+            fl = ctypes.c_double(0.0)
+            run = lambda: _abi.check(L.fsw_probe_mfma_mix(mix, 10000, 2 * ncu, p(window), window.numel(), p(sink), stream, ctypes.byref(fl)))  # noqa: E731
+            ms = gpu_time_ms(run, iters=3, warmup=1)
+            ceil[name] = round(fl.value / ms / 1e9, 1)
+        del window
         big = torch.empty(1 << 31, device=dev, dtype=torch.uint8).fill_(1)
         ms = gpu_time_ms(lambda: _abi.check(L.fsw_probe_stream_read(p(big), big.numel(), p(sink), stream)), iters=5, warmup=2)
         ceil["hbm_stream_read_gbs"] = round(big.numel() / ms / 1e6, 1)

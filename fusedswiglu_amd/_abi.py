@@ -34,6 +34,7 @@ EXPORTED_SYMBOLS = (
     "fsw_weight_grad",
     "fsw_probe_mfma",
     "fsw_probe_stream_read",
+    "fsw_probe_mfma_mix",
 )
 
 
@@ -108,6 +109,8 @@ def lib() -> ctypes.CDLL:
         L.fsw_probe_mfma.argtypes = [ci, ci, ci, vp, vp, ctypes.POINTER(ctypes.c_double)]
         L.fsw_probe_stream_read.restype = ci
         L.fsw_probe_stream_read.argtypes = [vp, i64, vp, vp]
+        L.fsw_probe_mfma_mix.restype = ci
+        L.fsw_probe_mfma_mix.argtypes = [ci, ci, ci, vp, i64, vp, vp, ctypes.POINTER(ctypes.c_double)]
         _lib = L
     return _lib
 

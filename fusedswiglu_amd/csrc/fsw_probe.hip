@@ -42,6 +42,66 @@ __global__ __launch_bounds__(512) void probe_mfma_kernel(float* sink, int iters,
   if (s == 12345.678f) sink[0] = s;  // keeps the loop alive; practically never true
 }
 
+// The tiled kernels' instruction mix without any of their dependencies: per 8 MFMAs (16x16x32, N(0,1)
+// operands held in registers) NR 16-byte LDS reads per lane and ND direct global->LDS loads of 1 KiB
+// per wave, the loads hitting L2 (the 32 CUs of an XCD walk one 8 MiB window).  LDS values are consumed
+// one iteration after they were read, so nothing ever waits for fresh data: what this loop sustains is
+// what the matrix cores deliver while that much data moves beside them.
+template <int NR, int ND>
+__global__ __launch_bounds__(512) void probe_mfma_mix_kernel(const char* src, unsigned src_bytes, float* sink, int iters) {
+  __shared__ __attribute__((aligned(1024))) char smem[64 * 1024];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  for (int i = tid; i < 64 * 1024 / 16; i += 512) {
+    u32x4 v;
+    for (int e = 0; e < 4; e++) v[e] = __float_as_uint(probe_normal(i * 4 + e, 7));
+    ((FSW_LDS u32x4*)smem)[i] = v;
+  }
+  __syncthreads();
+  bf16x8 a[8], b[4];
+  for (int f = 0; f < 8; f++)
+    for (int j = 0; j < 8; j++) a[f][j] = (__bf16)probe_normal(tid * 64 + f * 8 + j + blockIdx.x * 77777, 1);
+  for (int f = 0; f < 4; f++)
+    for (int j = 0; j < 8; j++) b[f][j] = (__bf16)(probe_normal(tid * 64 + f * 8 + j + blockIdx.x * 33333, 2) * 0.015625f);
+  f32x4 acc[4][8];
+  for (int x = 0; x < 4; x++)
+    for (int q = 0; q < 8; q++) acc[x][q] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const i32x4 rs = make_rsrc(src, src_bytes);
+  const unsigned lds_base = (unsigned)(uintptr_t)(FSW_LDS char*)smem;
+  const unsigned goff = ((blockIdx.x & 31) * 8 + wave) * 1024 + lane * 16;
+  u32x4 x0 = {0, 0, 0, 0};
+  u32x4 pending[4][NR > 0 ? NR : 1];
+  for (int x = 0; x < 4; x++)
+    for (int r = 0; r < (NR > 0 ? NR : 1); r++) pending[x][r] = x0;
+  for (int it = 0; it < iters; it++) {
+#pragma unroll
+    for (int x = 0; x < 4; x++) {
+#pragma unroll
+      for (int q = 0; q < 8; q++) acc[x][q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[x], a[q], acc[x][q], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int r = 0; r < NR; r++) {
+        x0 ^= pending[x][r];
+        pending[x][r] = *(const FSW_LDS u32x4*)(smem + ((wave * 4 + x) * 4096 + r * 1024 + lane * 16) % 65536);
+      }
+#pragma unroll
+      for (int d = 0; d < ND; d++) {
+        const unsigned voff = (goff + (unsigned)(it * 4 + x) * 262144u) % src_bytes;  // 16-byte aligned, < src_bytes
+        load16_to_lds(rs, voff, lds_base + ((wave * 4 + x) * 4096 + d * 1024) % 65536);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  for (int x = 0; x < 4; x++)
+    for (int r = 0; r < (NR > 0 ? NR : 1); r++) x0 ^= pending[x][r];
+  float s = __uint_as_float(x0[0] ^ x0[1] ^ x0[2] ^ x0[3]);
+  for (int x = 0; x < 4; x++)
+    for (int q = 0; q < 8; q++)
+      for (int r = 0; r < 4; r++) s += acc[x][q][r];
+  if (s == 12345.678f) sink[0] = s;
+}
+
 __global__ __launch_bounds__(256) void probe_read_kernel(const u32x4* __restrict__ p, size_t n16, unsigned* sink) {
   const size_t stride = (size_t)gridDim.x * blockDim.x;
   unsigned s = 0;
@@ -63,6 +123,27 @@ int fsw_probe_mfma(int random_operands, int iters, int workgroups, void* sink4, 
   if (!sink4 || iters <= 0 || workgroups <= 0) return FSW_ERR_BAD_SHAPE;
   fsw::probe_mfma_kernel<<<workgroups, 512, 0, (hipStream_t)stream>>>((float*)sink4, iters, random_operands);
   if (flop_out) *flop_out = (double)workgroups * 8.0 * iters * 8.0 * 32768.0;
+  return hipGetLastError() == hipSuccess ? FSW_OK : FSW_ERR_LAUNCH;
+}
+
+int fsw_probe_mfma_mix(int mix, int iters, int workgroups, const void* buf, int64_t bytes, void* sink4,
+                       void* stream, double* flop_out) {
+  // the window must hold whole 256 KiB strides and stay below the 2 GiB reach of the descriptor
+  if (!buf || !sink4 || iters <= 0 || workgroups <= 0 || bytes < (1 << 20) || bytes >= (1LL << 31) ||
+      (bytes & 0x3ffff) || ((uintptr_t)buf & 15))
+    return FSW_ERR_BAD_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  const char* src = (const char*)buf;
+  const unsigned n = (unsigned)bytes;
+  switch (mix) {
+    case 0: fsw::probe_mfma_mix_kernel<0, 0><<<workgroups, 512, 0, s>>>(src, n, (float*)sink4, iters); break;
+    case 1: fsw::probe_mfma_mix_kernel<3, 1><<<workgroups, 512, 0, s>>>(src, n, (float*)sink4, iters); break;
+    case 2: fsw::probe_mfma_mix_kernel<2, 1><<<workgroups, 512, 0, s>>>(src, n, (float*)sink4, iters); break;
+    case 3: fsw::probe_mfma_mix_kernel<3, 0><<<workgroups, 512, 0, s>>>(src, n, (float*)sink4, iters); break;
+    case 4: fsw::probe_mfma_mix_kernel<0, 1><<<workgroups, 512, 0, s>>>(src, n, (float*)sink4, iters); break;
+    default: return FSW_ERR_BAD_SHAPE;
+  }
+  if (flop_out) *flop_out = (double)workgroups * 8.0 * iters * 32.0 * 16384.0;
   return hipGetLastError() == hipSuccess ? FSW_OK : FSW_ERR_LAUNCH;
 }
 
