@@ -85,6 +85,18 @@ def test_backward_validation(L):
     assert L.fsw_workspace_bytes(0, 8192, 256, 768) == 0 and L.fsw_workspace_bytes(1, 0, 1, 1) == 0
 
 
+def test_probe_validation(L):
+    f = L.fsw_probe_mfma_mix
+    flop = ctypes.c_double(0.0)
+    assert f(1, 10, 256, None, 8 << 20, P, None, ctypes.byref(flop)) == 3          # no source window
+    assert f(1, 10, 256, P, (8 << 20) + 4096, P, None, ctypes.byref(flop)) == 3    # not a multiple of 256 KiB
+    assert f(1, 10, 256, P, 1 << 31, P, None, ctypes.byref(flop)) == 3             # beyond the descriptor's reach
+    assert f(9, 10, 256, P, 8 << 20, P, None, ctypes.byref(flop)) == 3             # unknown mix
+    assert f(1, 0, 256, P, 8 << 20, P, None, ctypes.byref(flop)) == 3
+    assert L.fsw_probe_mfma(1, 0, 256, P, None, ctypes.byref(flop)) == 3
+    assert L.fsw_probe_stream_read(None, 1 << 20, P, None) == 3
+
+
 def test_kernel_selection_logic(L):
     t = L.fsw_uses_tiled_kernel
     # the north-star shape and the fp16 config run on the tiled kernels in all three steps
