@@ -6,12 +6,16 @@
 //
 // One workgroup = 8 wavefronts (4 along M x 2 along N) = one 256 x 256 fp32 accumulator tile
 // (kFwd / kDw: 256 rows x 128 columns of EACH of the two results, sharing the A tile).
-// The reduction advances 32 elements per step.  Operand tiles are brought in by direct
-// global->LDS loads several steps ahead of the MFMAs and kept in LDS rings:
-//   * an m/n-contiguous ("MC") operand uses a ring of four 16 KiB slots, one per step;
+// The reduction advances 32 elements per step and is organised in PAIRS of steps.  Operand tiles are
+// brought in by direct global->LDS loads one to two pairs ahead of the MFMAs and kept in LDS rings
+// (A: three pairs, B: two pairs, 160 KiB in all):
+//   * an m/n-contiguous ("MC") operand uses 16 KiB slots, one per step;
 //   * a k-contiguous ("KC") operand is fetched 64 k-elements (one full 128-byte line per row) at a
-//     time into a ring of 32 KiB areas, each serving two consecutive steps.  Fetching half lines
+//     time into 32 KiB areas, each serving the two steps of a pair.  Fetching half lines
 //     (64 bytes per row per step) halves the throughput of the texture-address path.
+// Every wave runs the same free-running loop: it holds the fragments of BOTH steps of the current pair
+// in registers, so a pair's LDS space is released (and refilled) at the single barrier in the middle of
+// the pair, and the fragment reads of a step are always one step ahead of the MFMAs that consume them.
 #pragma once
 #include "fsw_common.hpp"
 
@@ -42,7 +46,6 @@ struct GemmParams {
 
 constexpr int kThreads = 512;
 constexpr int kTileM = 256;
-constexpr int kMcSlots = 4;
 constexpr int kMcSlotBytes = 2 * kMcPanelBytes;  // two 128-column panels: 16 KiB
 constexpr int kKcAreaBytes = 256 * 128;          // 256 rows x 64 k-elements: 32 KiB
 
@@ -51,16 +54,13 @@ struct Cfg {
   static constexpr bool kAKc = (MODE != kDw);
   static constexpr bool kBKc = (MODE == kDx);
   static constexpr int kTileN = (MODE == kDx) ? 256 : 128;
-  // KC rings: number of 32 KiB areas.  160 KiB of LDS in all for kFwd and kDx, 128 KiB for kDw.
-  static constexpr int kAreasA = 3;
-  static constexpr int kAreasB = 2;
-  static constexpr int kBytesA = kAKc ? kAreasA * kKcAreaBytes : kMcSlots * kMcSlotBytes;
-  static constexpr int kBytesB = kBKc ? kAreasB * kKcAreaBytes : kMcSlots * kMcSlotBytes;
-  // how many steps ahead of its use an operand's loads are issued
-  static constexpr int kAheadA = kAKc ? 2 * (kAreasA - 1) : kMcSlots - 1;
-  static constexpr int kAheadB = kBKc ? 2 * (kAreasB - 1) : kMcSlots - 1;
-  static constexpr int kAheadMax = kAheadA > kAheadB ? kAheadA : kAheadB;
+  // rings in pairs of steps: 96 KiB for A, 64 KiB for B in either layout
+  static constexpr int kPairsA = 3;
+  static constexpr int kPairsB = 2;
+  static constexpr int kBytesA = kPairsA * kKcAreaBytes;
+  static constexpr int kBytesB = kPairsB * kKcAreaBytes;
 };
+static_assert(kKcAreaBytes == 2 * kMcSlotBytes, "a pair of steps takes 32 KiB in either layout");
 
 // ---- fragment reads -----------------------------------------------------------
 // KC area: 256 rows x 128 bytes; the 16-byte chunk c of row r sits at chunk position
@@ -188,55 +188,57 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
   if constexpr (B_KC) kc_setup(kb, p.b0, p.b1, n0, p.N, p.K, p.ldb, wave, lane);
   else mc_setup(mb, p.b0, p.b1, n0, n0, p.N, p.K, p.ldb, wave, lane);
 
-  // loads of the pair of steps (pr, pr+1) of a KC operand into area (pr/2) % areas
-  auto issue_kc = [&](const KcLoader& L, int pr, int areas, unsigned lds_base) {
-    if (pr < 0 || pr >= kt_total) return;
-    const int apr = kbase + pr;  // absolute step
+  // Loads of the pair of steps (st, st+1), st even: four 1 KiB instructions per wave in either layout.
+  // They are issued for EVERY pair index the loop asks for, also beyond the end of the reduction, where
+  // every lane is out of range and zero-fills: the loop below is branch-free and its vmcnt arithmetic
+  // never changes (and a last, odd step is multiplied by zeros).
+  auto kc_pair = [&](const KcLoader& L, int st, int pairs, unsigned lds_base) {
+    const int apr = kbase + st;  // absolute step
     const int pass = (MODE == kDx && apr >= kt1) ? 1 : 0;
     const int k0 = (apr - pass * kt1) * kBK;
     const i32x4 rs = make_rsrc((pass ? L.base1 : L.base0) + (size_t)k0 * 2);
-    const unsigned dst = lds_base + (unsigned)((pr >> 1) % areas) * kKcAreaBytes + wave * 1024;
+    const unsigned dst = lds_base + (unsigned)((st >> 1) % pairs) * kKcAreaBytes + wave * 1024;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const unsigned off = (k0 < L.klim[i]) ? L.lane_off + i * L.row_step : kOobOffset;
       load16_to_lds(rs, off, dst + i * 8192);
     }
   };
-  // loads of step s of an MC operand into slot s % 4
-  auto issue_mc = [&](const McLoader& L, int s, unsigned lds_base) {
-    if (s < 0 || s >= kt_total) return;
-    const int k0 = (kbase + s) * kBK;
-    const unsigned dst = lds_base + (unsigned)(s & (kMcSlots - 1)) * kMcSlotBytes + wave * 1024;
+  auto mc_step = [&](const McLoader& L, int st, int pairs, unsigned lds_base) {
+    const int k0 = (kbase + st) * kBK;
+    const unsigned dst = lds_base + (unsigned)(st % (2 * pairs)) * kMcSlotBytes + wave * 1024;
 #pragma unroll
     for (int i = 0; i < 2; i++) {
       const unsigned off = (k0 < L.klim[i]) ? L.lane_off[i] : kOobOffset;
-      load16_to_lds(make_rsrc(L.base[i] + (size_t)(kbase + s) * L.kstep), off, dst + i * 8192);
+      load16_to_lds(make_rsrc(L.base[i] + (size_t)(kbase + st) * L.kstep), off, dst + i * 8192);
     }
   };
-  // everything a wave issues during step i (i < 0: prologue).  The order fixes the vmcnt arithmetic below.
-  auto issue_step = [&](int i) {
-    if ((i & 1) == 0) {
-      if constexpr (B_KC) issue_kc(kb, i + C::kAheadB, C::kAreasB, smem_b);
-      if constexpr (A_KC) issue_kc(ka, i + C::kAheadA, C::kAreasA, smem_a);
-    }
-    if constexpr (!A_KC) issue_mc(ma, i + C::kAheadA, smem_a);
-    if constexpr (!B_KC) issue_mc(mb, i + C::kAheadB, smem_b);
+  auto issue_a = [&](int st) {
+    if constexpr (A_KC) kc_pair(ka, st, C::kPairsA, smem_a);
+    else { mc_step(ma, st, C::kPairsA, smem_a); mc_step(ma, st + 1, C::kPairsA, smem_a); }
   };
-  // Wait until this wave's share of step kt+1 has landed, then meet the other waves.  Loads complete in
-  // issue order, so it is enough to bound how many of the younger ones may still be in flight:
-  //   kFwd  after the MC slot of step kt+1 (issued during step kt-2) come one KC batch (4) and two MC
-  //         batches (2+2)                                                                    -> 8
-  //   kDw   two steps of 2+2                                                                 -> 8
-  //   kDx   step kt odd: after the B pair of kt+1 (issued first during step kt-1) comes only the A pair
-  //         issued with it -> 4;  kt even: nothing new is needed, this step's 8 loads are younger -> 12
-  // Near the end of the reduction, where some of those loads no longer exist, wait for everything.
-  auto wait_next_step_and_barrier = [&](int kt) {
-    if (kt + C::kAheadMax >= kt_total) { wait_vmcnt_and_barrier<0>(); return; }
-    if constexpr (MODE == kDx) {
-      if (kt & 1) wait_vmcnt_and_barrier<4>();
-      else wait_vmcnt_and_barrier<12>();
-    } else {
-      wait_vmcnt_and_barrier<8>();
+  auto issue_b = [&](int st) {
+    if constexpr (B_KC) kc_pair(kb, st, C::kPairsB, smem_b);
+    else { mc_step(mb, st, C::kPairsB, smem_b); mc_step(mb, st + 1, C::kPairsB, smem_b); }
+  };
+  // the 4 + 8 fragments of step kt (reading beyond the last step returns stale LDS bytes nobody uses)
+  auto read_frags = [&](int kt, i16x8 (&fq)[4], i16x8 (&fp)[8]) {
+    const FSW_LDS char* ra;
+    const FSW_LDS char* rb;
+    if constexpr (A_KC) ra = lds_a + ((kt >> 1) % C::kPairsA) * kKcAreaBytes;
+    else ra = lds_a + (kt % (2 * C::kPairsA)) * kMcSlotBytes;
+    if constexpr (B_KC) rb = lds_b + ((kt >> 1) % C::kPairsB) * kKcAreaBytes;
+    else rb = lds_b + (kt % (2 * C::kPairsB)) * kMcSlotBytes;
+    const int half = kt & 1;
+#pragma unroll
+    for (int mb = 0; mb < 4; mb++) {
+      if constexpr (A_KC) fq[mb] = read_frag_kc16(ra, wm * 64 + mb * 16, half, lane);
+      else fq[mb] = read_frag_mc16(ra + (wm >> 1) * kMcPanelBytes, (wm & 1) * 4 + mb, lane);
+    }
+#pragma unroll
+    for (int nb = 0; nb < 8; nb++) {
+      if constexpr (B_KC) fp[nb] = read_frag_kc16(rb, wn * 128 + nb * 16, half, lane);
+      else fp[nb] = read_frag_mc16(rb + (nb >> 2) * kMcPanelBytes, wn * 4 + (nb & 3), lane);
     }
   };
 
@@ -248,53 +250,50 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
   for (int nb = 0; nb < 8; nb++)
 #pragma unroll
     for (int mb = 0; mb < 4; mb++) acc[nb][mb] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-  // ---- main loop: two groups of four waves (one per SIMD each) run half a step out of phase.
-  // While one group reads its fragments of a step from LDS (and issues its share of the loads for
-  // later steps), the other group issues the 32 MFMAs of the step it read one phase earlier, so the
-  // matrix cores of every SIMD always have a wave to serve.  Phases are separated by workgroup
-  // barriers; group 1 enters one barrier late, group 0 makes up for it after the loop.
-  const int grp = wave >> 2;
-#pragma unroll
-  for (int i = -C::kAheadMax; i < 0; i++) issue_step(i);
-  wait_next_step_and_barrier(-1);
-  if (grp == 1) wait_vmcnt_and_barrier<63>();
-
-  for (int kt = 0; kt < kt_total; kt++) {
-    const FSW_LDS char* ra;
-    const FSW_LDS char* rb;
-    if constexpr (A_KC) ra = lds_a + ((kt >> 1) % C::kAreasA) * kKcAreaBytes;
-    else ra = lds_a + (kt & (kMcSlots - 1)) * kMcSlotBytes;
-    if constexpr (B_KC) rb = lds_b + ((kt >> 1) % C::kAreasB) * kKcAreaBytes;
-    else rb = lds_b + (kt & (kMcSlots - 1)) * kMcSlotBytes;
-    const int half = kt & 1;
-    i16x8 fq[4], fp[8];
-#pragma unroll
-    for (int mb = 0; mb < 4; mb++) {
-      if constexpr (A_KC) fq[mb] = read_frag_kc16(ra, wm * 64 + mb * 16, half, lane);
-      else fq[mb] = read_frag_mc16(ra + (wm >> 1) * kMcPanelBytes, (wm & 1) * 4 + mb, lane);
-    }
-#pragma unroll
-    for (int nb = 0; nb < 8; nb++) {
-      if constexpr (B_KC) fp[nb] = read_frag_kc16(rb, wn * 128 + nb * 16, half, lane);
-      else fp[nb] = read_frag_mc16(rb + (nb >> 2) * kMcPanelBytes, wn * 4 + (nb & 3), lane);
-    }
-    issue_step(kt);
-    wait_next_step_and_barrier(kt);
+  // 16 of a step's 32 MFMAs; consecutive MFMAs share one operand (the m index snakes back and forth)
+  auto mfma_half = [&](const i16x8 (&fq)[4], const i16x8 (&fp)[8], int h) {
     __builtin_amdgcn_sched_barrier(0);
-    // consecutive MFMAs share one operand (the m index snakes back and forth)
 #pragma unroll
-    for (int nb = 0; nb < 8; nb++)
+    for (int nb = 4 * h; nb < 4 * h + 4; nb++)
 #pragma unroll
       for (int i = 0; i < 4; i++) {
         const int mb = (nb & 1) ? 3 - i : i;
         acc[nb][mb] = E::mfma16(fp[nb], fq[mb], acc[nb][mb]);
       }
     __builtin_amdgcn_sched_barrier(0);
-    wait_vmcnt_and_barrier<63>();
+  };
+  // The barrier in the middle of pair p.  Before it a wave waits until everything it loaded except the
+  // four instructions of A(p+2), issued in this pair's first half, has landed - that includes its share of
+  // pair p+1 - and until its own fragment reads of pair p have returned; after it every wave may read pair
+  // p+1 and overwrite pair p's LDS space.
+  auto mid_barrier = [&]() { asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+
+  // ---- main loop, per pair p of steps (kt = 2p, fragments of step kt already on their way to registers):
+  //   first half   issue A(p+2) (its ring space, pair p-1, was released at the last barrier);
+  //                read the fragments of step kt+1;  32 MFMAs of step kt
+  //   barrier      (see mid_barrier)
+  //   second half  issue B(p+2) into pair p's space;  read the fragments of step kt+2;  32 MFMAs of kt+1
+  // The two waves of a SIMD (wave and wave + 4) meet that barrier half an MFMA block apart, so they never
+  // issue their loads and fragment reads at the same moment and the matrix core always has work queued.
+  const int grp = wave >> 2;
+  issue_a(0); issue_b(0); issue_a(2); issue_b(2);
+  wait_vmcnt_and_barrier<8>();
+  i16x8 fq0[4], fp0[8], fq1[4], fp1[8];
+  read_frags(0, fq0, fp0);
+  for (int kt = 0; kt < kt_total; kt += 2) {
+    issue_a(kt + 4);
+    read_frags(kt + 1, fq1, fp1);
+    mfma_half(fq0, fp0, 0);
+    if (grp == 1) mid_barrier();
+    mfma_half(fq0, fp0, 1);
+    if (grp == 0) mid_barrier();
+    issue_b(kt + 4);
+    read_frags(kt + 2, fq0, fp0);
+    mfma_half(fq1, fp1, 0);
+    mfma_half(fq1, fp1, 1);
   }
-  if (grp == 0) wait_vmcnt_and_barrier<63>();
-  // Every wave has passed its last read of the operand rings and every load has landed: LDS is free.
+  // the zero-filling loads beyond the end must have landed before the epilogue reuses LDS
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
   // ---- epilogue.  acc[nb][mb][r] of lane l is row  wm*64 + mb*16 + (l & 15)  of the tile and column
   // cbase(nb) + 4*(l >> 4) + r.  Each wave owns 64 consecutive columns (128 bytes) per result row, so
