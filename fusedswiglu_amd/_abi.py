@@ -19,6 +19,10 @@ DTYPE_FP16 = 1
 
 STEP_FORWARD, STEP_INPUT_GRAD, STEP_WEIGHT_GRAD = 0, 1, 2
 
+#: size of the scratch built into the library for fsw_input_grad_noalloc (FSW_NOALLOC_SCRATCH_BYTES)
+NOALLOC_SCRATCH_BYTES = 32 << 20
+ERR_SCRATCH_LIMIT = 7
+
 #: every symbol include/fusedswiglu.h declares
 EXPORTED_SYMBOLS = (
     "fsw_version",
@@ -31,6 +35,7 @@ EXPORTED_SYMBOLS = (
     "fsw_elementwise_backward",
     "fsw_gating_grad_recompute",
     "fsw_input_grad",
+    "fsw_input_grad_noalloc",
     "fsw_weight_grad",
     "fsw_probe_mfma",
     "fsw_probe_stream_read",
@@ -101,6 +106,8 @@ def lib() -> ctypes.CDLL:
         L.fsw_gating_grad_recompute.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, vp]
         L.fsw_input_grad.restype = ci
         L.fsw_input_grad.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, i64, ci, vp]
+        L.fsw_input_grad_noalloc.restype = ci
+        L.fsw_input_grad_noalloc.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, vp]
         L.fsw_weight_grad.restype = ci
         L.fsw_weight_grad.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, i64, ci, vp]
         L.fsw_workspace_bytes.restype = i64

@@ -4,6 +4,7 @@
 #include <atomic>
 #include <cstdarg>
 #include <cstdio>
+#include <mutex>
 
 namespace {
 
@@ -58,6 +59,7 @@ const char* fsw_status_string(int status) {
     case FSW_ERR_BAD_STRIDE: return "bad leading dimension";
     case FSW_ERR_ALIGNMENT: return "pointer not 2-byte aligned";
     case FSW_ERR_LAUNCH: return "kernel launch failed";
+    case FSW_ERR_SCRATCH_LIMIT: return "problem needs more scratch than the built-in buffer holds";
     default: return "unknown status";
   }
 }
@@ -148,11 +150,9 @@ int fsw_elementwise_backward(const void* grad_out, const void* xw_gate, const vo
                                               (size_t)numel, (hipStream_t)stream));
 }
 
-int fsw_input_grad(const void* grad_xw_gate, const void* grad_xw_up, const void* w_gate,
-                   const void* w_up, void* grad_x, int64_t T, int64_t D, int64_t I, int64_t ldo,
-                   int64_t ldw, int64_t ld_dx, void* workspace, int64_t workspace_bytes, int dtype,
-                   void* stream) {
-  const char* fn = "fsw_input_grad";
+static int check_input_grad_args(const char* fn, const void* grad_xw_gate, const void* grad_xw_up,
+                                 const void* w_gate, const void* w_up, void* grad_x, int64_t T, int64_t D,
+                                 int64_t I, int64_t ldo, int64_t ldw, int64_t ld_dx, int dtype) {
   if (!grad_xw_gate || !grad_xw_up || !w_gate || !w_up || !grad_x)
     return fail(FSW_ERR_NULL_POINTER, "%s: all five arrays must be non-null", fn);
   if (!dtype_ok(dtype)) return fail(FSW_ERR_BAD_DTYPE, "%s: dtype %d is neither bf16 (0) nor fp16 (1)", fn, dtype);
@@ -162,6 +162,13 @@ int fsw_input_grad(const void* grad_xw_gate, const void* grad_xw_up, const void*
   if (int e = check_ld(fn, "ld_dx", ld_dx, D)) return e;
   if (!al2(grad_xw_gate) || !al2(grad_xw_up) || !al2(w_gate) || !al2(w_up) || !al2(grad_x))
     return fail(FSW_ERR_ALIGNMENT, "%s: pointers must be 2-byte aligned", fn);
+  return FSW_OK;
+}
+
+static int input_grad_checked(const char* fn, const void* grad_xw_gate, const void* grad_xw_up,
+                              const void* w_gate, const void* w_up, void* grad_x, int64_t T, int64_t D,
+                              int64_t I, int64_t ldo, int64_t ldw, int64_t ld_dx, void* workspace,
+                              int64_t workspace_bytes, int dtype, void* stream) {
   fsw::Problem p{};
   p.dG = grad_xw_gate; p.dU = grad_xw_up; p.wg = w_gate; p.wu = w_up; p.dx = grad_x;
   p.T = T; p.D = D; p.I = I; p.ldo = ldo; p.ldw = ldw; p.lddx = ld_dx;
@@ -171,6 +178,17 @@ int fsw_input_grad(const void* grad_xw_gate, const void* grad_xw_up, const void*
     return launched(fn, fsw::launch_input_grad_fast(dtype, p, s, ws_ok ? workspace : nullptr, ws_ok ? workspace_bytes : 0));
   }
   return launched(fn, fsw::launch_input_grad_generic(dtype, p, s));
+}
+
+int fsw_input_grad(const void* grad_xw_gate, const void* grad_xw_up, const void* w_gate,
+                   const void* w_up, void* grad_x, int64_t T, int64_t D, int64_t I, int64_t ldo,
+                   int64_t ldw, int64_t ld_dx, void* workspace, int64_t workspace_bytes, int dtype,
+                   void* stream) {
+  const char* fn = "fsw_input_grad";
+  if (int e = check_input_grad_args(fn, grad_xw_gate, grad_xw_up, w_gate, w_up, grad_x, T, D, I, ldo, ldw, ld_dx, dtype))
+    return e;
+  return input_grad_checked(fn, grad_xw_gate, grad_xw_up, w_gate, w_up, grad_x, T, D, I, ldo, ldw, ld_dx,
+                            workspace, workspace_bytes, dtype, stream);
 }
 
 int fsw_weight_grad(const void* x, const void* grad_xw_up, const void* grad_xw_gate,
@@ -196,6 +214,59 @@ int fsw_weight_grad(const void* x, const void* grad_xw_up, const void* grad_xw_g
     return launched(fn, fsw::launch_weight_grad_fast(dtype, p, s, ws_ok ? workspace : nullptr, ws_ok ? workspace_bytes : 0));
   }
   return launched(fn, fsw::launch_weight_grad_generic(dtype, p, s));
+}
+
+// ---- the entry point that allocates nothing -------------------------------------------------
+// Scratch for the split reduction of fsw_input_grad_noalloc: one copy per GPU, part of the library's
+// code object, held until the process ends.  In host code `scratch` is only a handle; the device
+// address is looked up once per device with hipGetSymbolAddress and kept in g_scratch_ptr.
+static __device__ __align__(256) unsigned char scratch[FSW_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of this device's copy of `scratch` (nullptr + message on failure).
+void* scratch_address(const char* fn) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    fail(FSW_ERR_LAUNCH, "%s: hipGetDevice failed or device index %d is beyond %d", fn, dev, kMaxDevices);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      fail(FSW_ERR_LAUNCH, "%s: hipGetSymbolAddress(scratch): %s", fn, hipGetErrorString(e));
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = ptr;
+  }
+  return g_scratch_ptr[dev];
+}
+}  // namespace
+
+int fsw_input_grad_noalloc(const void* grad_xw_gate, const void* grad_xw_up, const void* w_gate,
+                           const void* w_up, void* grad_x, int64_t T, int64_t D, int64_t I, int64_t ldo,
+                           int64_t ldw, int64_t ld_dx, int dtype, void* stream) {
+  const char* fn = "fsw_input_grad_noalloc";
+  if (int e = check_input_grad_args(fn, grad_xw_gate, grad_xw_up, w_gate, w_up, grad_x, T, D, I, ldo, ldw, ld_dx, dtype))
+    return e;
+  const int64_t need = fsw::splitk_workspace_bytes(1, T, D, I);
+  if (need > (int64_t)FSW_NOALLOC_SCRATCH_BYTES)
+    return fail(FSW_ERR_SCRATCH_LIMIT,
+                "%s: T=%lld D=%lld I=%lld needs %lld bytes of split-reduction scratch, the built-in buffer holds %lld; "
+                "use fsw_input_grad with a caller workspace",
+                fn, (long long)T, (long long)D, (long long)I, (long long)need, (long long)FSW_NOALLOC_SCRATCH_BYTES);
+  void* ptr = scratch_address(fn);
+  if (!ptr) return FSW_ERR_LAUNCH;
+  // Every partial the reduction kernel reads is written by the GEMM kernel of the same call, so nothing in
+  // the buffer has to start at zero.
+  return input_grad_checked(fn, grad_xw_gate, grad_xw_up, w_gate, w_up, grad_x, T, D, I, ldo, ldw, ld_dx, ptr,
+                            (int64_t)FSW_NOALLOC_SCRATCH_BYTES, dtype, stream);
 }
 
 }  // extern "C"

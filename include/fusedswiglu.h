@@ -46,7 +46,8 @@ enum {
   FSW_ERR_BAD_SHAPE = 3,  /* a dimension is <= 0 or exceeds 2^31-1 */
   FSW_ERR_BAD_STRIDE = 4, /* a leading dimension is smaller than the row it describes */
   FSW_ERR_ALIGNMENT = 5,  /* a pointer is not 2-byte aligned */
-  FSW_ERR_LAUNCH = 6      /* the HIP runtime refused the launch; see fsw_last_error() */
+  FSW_ERR_LAUNCH = 6,     /* the HIP runtime refused the launch; see fsw_last_error() */
+  FSW_ERR_SCRATCH_LIMIT = 7 /* fsw_input_grad_noalloc: the problem needs more than FSW_NOALLOC_SCRATCH_BYTES */
 };
 
 /* Library version (FSW_VERSION it was built with). */
@@ -117,6 +118,22 @@ int fsw_input_grad(const void* grad_xw_gate, const void* grad_xw_up, const void*
                    const void* w_up, void* grad_x, int64_t T, int64_t D, int64_t I, int64_t ldo,
                    int64_t ldw, int64_t ld_dx, void* workspace, int64_t workspace_bytes, int dtype,
                    void* stream);
+
+/*
+ * fsw_input_grad for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same
+ * arguments and results as fsw_input_grad, but the fp32 scratch of the split reduction is a buffer of
+ * FSW_NOALLOC_SCRATCH_BYTES built into the library (one copy per GPU, held until the process ends)
+ * instead of a caller workspace; the call itself allocates and frees nothing.  Problems whose
+ * fsw_workspace_bytes(1, T, D, I) exceeds that size are rejected with FSW_ERR_SCRATCH_LIMIT (large
+ * problems need no scratch at all and always pass).  All calls on one GPU share that GPU's buffer:
+ * calls that overlap in time on one GPU (different streams or threads) race on it.  The first call
+ * on a device looks the buffer's address up; make that call outside graph capture.
+ */
+#define FSW_NOALLOC_SCRATCH_BYTES (32u << 20)
+int fsw_input_grad_noalloc(const void* grad_xw_gate, const void* grad_xw_up, const void* w_gate,
+                           const void* w_up, void* grad_x, int64_t T, int64_t D, int64_t I, int64_t ldo,
+                           int64_t ldw, int64_t ld_dx, int dtype, void* stream);
 
 /*
  * Weight gradients: grad_w_gate = x^T grad_xw_gate, grad_w_up = x^T grad_xw_up, reduced over

@@ -34,8 +34,8 @@ def test_header_symbols_all_exported(L):
 
 def test_status_strings(L):
     assert L.fsw_status_string(0) == b"ok"
-    seen = {L.fsw_status_string(i) for i in range(0, 7)}
-    assert len(seen) == 7
+    seen = {L.fsw_status_string(i) for i in range(0, 8)}
+    assert len(seen) == 8
     assert L.fsw_status_string(99) == b"unknown status"
 
 
@@ -73,6 +73,17 @@ def test_backward_validation(L):
     assert dx(P, P, P, P, None, 8, 8, 8, 8, 8, 8, None, 0, 0, None) == 1
     assert dx(P, P, P, P, P, 8, 8, 8, 8, 8, 4, None, 0, 0, None) == 4  # ld_dx < D
     assert dx(P, P, P, P, P, 8, 8, 0, 8, 8, 8, None, 0, 0, None) == 3
+    # the variant on the library's built-in scratch validates the same way, and turns problems whose split
+    # reduction needs more than that buffer away before it touches the GPU
+    na = L.fsw_input_grad_noalloc
+    assert na(P, P, P, P, None, 8, 8, 8, 8, 8, 8, 0, None) == 1
+    assert na(P, P, P, P, P, 8, 8, 8, 8, 8, 4, 0, None) == 4
+    assert na(P, P, P, P, P, 8, 8, 8, 8, 8, 8, 9, None) == 2
+    assert L.fsw_workspace_bytes(1, 16384, 256, 2048) > _abi.NOALLOC_SCRATCH_BYTES
+    assert na(P, P, P, P, P, 16384, 256, 2048, 2048, 2048, 256, 0, None) == _abi.ERR_SCRATCH_LIMIT
+    assert b"built-in buffer" in L.fsw_last_error()
+    header = open(os.path.join(ROOT, "include", "fusedswiglu.h")).read()
+    assert re.search(r"#define FSW_NOALLOC_SCRATCH_BYTES \(32u << 20\)", header) and _abi.NOALLOC_SCRATCH_BYTES == 32 << 20
     dw = L.fsw_weight_grad
     assert dw(P, None, P, P, P, 8, 8, 8, 8, 8, 8, None, 0, 1, None) == 1
     assert dw(P, P, P, P, P, 8, 8, 8, 8, 8, 8, None, 0, -3, None) == 2
