@@ -22,9 +22,11 @@ NAME = {torch.bfloat16: "bf16", torch.float16: "fp16"}
 FUNC = {torch.bfloat16: FusedSwiGLU, torch.float16: FastAccumFusedSwiGLU}
 KERN = {torch.bfloat16: kernels_bf16, torch.float16: kernels_fp16}
 try:
-    NUM_TEST = int(os.environ["NUM_TEST"])  # same knob as test_swiglu.py:13-16
+    # the upstream knob (test_swiglu.py:13-16), kept as an optional reducer: NUM_TEST=2 runs 16 + 16 of the
+    # reference's 81 + 81 cases.  The default runs all of them, in both element types.
+    NUM_TEST = int(os.environ["NUM_TEST"])
 except Exception:
-    NUM_TEST = 3
+    NUM_TEST = None
 
 
 def np64(t: torch.Tensor) -> np.ndarray:
@@ -159,8 +161,10 @@ def _grid_cases(kind):
     here = os.path.dirname(os.path.abspath(__file__))
     with open(os.path.join(here, "golden", "reference_shape_grid.json")) as f:
         cases = json.load(f)[kind]
-    # NUM_TEST controls breadth like upstream: NUM_TEST**2 cases spread over the 81
-    n = min(len(cases), NUM_TEST ** 2)
+    if NUM_TEST is None:
+        return [tuple(c) for c in cases]
+    # NUM_TEST**4 cases spread over the 81, as upstream's four nested draws would give
+    n = max(1, min(len(cases), NUM_TEST ** 4))
     idx = np.linspace(0, len(cases) - 1, n).round().astype(int)
     return [tuple(cases[i]) for i in idx]
 
@@ -192,30 +196,38 @@ def _slice_check(oracle, dtype, tx, twg, twu, tdy, out, dx, dwg, dwu, n_rows=6, 
     return errs
 
 
-@pytest.mark.parametrize("dims", _grid_cases("fwd"), ids=lambda s: "x".join(map(str, s)))
-def test_reference_grid_forward(oracle, dims):
-    """The forward cases of the reference's test (test_swiglu.py:58-78), bf16, under no_grad."""
-    B, S, D, I = dims
-    g = torch.Generator(device=DEV).manual_seed(0)
-    tx = torch.randn(B, S, D, device=DEV, dtype=torch.bfloat16, generator=g)
-    twg = torch.randn(D, I, device=DEV, dtype=torch.bfloat16, generator=g) / D ** 0.5
-    twu = torch.randn(D, I, device=DEV, dtype=torch.bfloat16, generator=g) / D ** 0.5
+def _grid_id(case):
+    return f"{case[0]:02d}-" + "x".join(map(str, case[1]))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("case", list(enumerate(_grid_cases("fwd"))), ids=_grid_id)
+def test_reference_grid_forward(oracle, case, dtype):
+    """The forward cases of the reference's test (test_swiglu.py:58-78) under no_grad: all 81 shapes, in bf16
+    through FusedSwiGLU as upstream and in fp16 through FastAccumFusedSwiGLU (untested upstream)."""
+    B, S, D, I = case[1]
+    g = torch.Generator(device=DEV).manual_seed(case[0])
+    tx = torch.randn(B, S, D, device=DEV, dtype=dtype, generator=g)
+    twg = torch.randn(D, I, device=DEV, dtype=dtype, generator=g) / D ** 0.5
+    twu = torch.randn(D, I, device=DEV, dtype=dtype, generator=g) / D ** 0.5
     with torch.no_grad():
-        out = FusedSwiGLU.apply(tx, twg, twu)
-    _slice_check(oracle, torch.bfloat16, tx, twg, twu, None, out, None, None, None)
+        out = FUNC[dtype].apply(tx, twg, twu)
+    _slice_check(oracle, dtype, tx, twg, twu, None, out, None, None, None, n_rows=3, seed=case[0])
 
 
-@pytest.mark.parametrize("dims", _grid_cases("bwd"), ids=lambda s: "x".join(map(str, s)))
-def test_reference_grid_backward(oracle, dims):
-    """The backward cases of the reference's test (test_swiglu.py:81-114): dy = 0.1 * randn."""
-    B, S, D, I = dims
-    g = torch.Generator(device=DEV).manual_seed(0)
-    tx = torch.randn(B, S, D, device=DEV, dtype=torch.bfloat16, generator=g)
-    twg = torch.randn(D, I, device=DEV, dtype=torch.bfloat16, generator=g) / D ** 0.5
-    twu = torch.randn(D, I, device=DEV, dtype=torch.bfloat16, generator=g) / D ** 0.5
-    tdy = 0.1 * torch.randn(B, S, I, device=DEV, dtype=torch.bfloat16, generator=g)
-    out, dx, dwg, dwu = run_fwd_bwd(torch.bfloat16, tx, twg, twu, tdy)
-    _slice_check(oracle, torch.bfloat16, tx, twg, twu, tdy, out, dx, dwg, dwu)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("case", list(enumerate(_grid_cases("bwd"))), ids=_grid_id)
+def test_reference_grid_backward(oracle, case, dtype):
+    """The backward cases of the reference's test (test_swiglu.py:81-114), dy = 0.1 * randn: all 81 shapes in
+    both element types; out, dx, dWg and dWu are each held to the bound."""
+    B, S, D, I = case[1]
+    g = torch.Generator(device=DEV).manual_seed(case[0])
+    tx = torch.randn(B, S, D, device=DEV, dtype=dtype, generator=g)
+    twg = torch.randn(D, I, device=DEV, dtype=dtype, generator=g) / D ** 0.5
+    twu = torch.randn(D, I, device=DEV, dtype=dtype, generator=g) / D ** 0.5
+    tdy = 0.1 * torch.randn(B, S, I, device=DEV, dtype=dtype, generator=g)
+    out, dx, dwg, dwu = run_fwd_bwd(dtype, tx, twg, twu, tdy)
+    _slice_check(oracle, dtype, tx, twg, twu, tdy, out, dx, dwg, dwu, n_rows=3, n_cols=3, seed=case[0])
 
 
 FULL = {
