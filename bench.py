@@ -22,15 +22,41 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16/fp16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
-# HBM-side bytes per launch (L2 <-> fabric reads + writes) of the three GEMM kernels at the C2 shape,
-# from the FETCH_SIZE / WRITE_SIZE counter passes summarised in profiles/gemm_kernels_c2_bf16.md
-# (FETCH_SIZE scaled by 2.0, WRITE_SIZE by 1.0 against a plain 1 GiB copy).  bench.py cannot run the
-# profiler itself; this table is refreshed whenever that profile is.
-PROFILED_TRAFFIC_BYTES = {
-    "forward_dual_gemm": (2 * 1180115 + 589824) * 1024,
-    "input_grad_dual_gemm": (2 * 1180438 + 65536) * 1024,
-    "weight_grad_dual_gemm": (2 * 1179789 + 196608) * 1024,
-}
+# HBM-side bytes per launch (L2 <-> fabric reads + writes) of the three GEMM kernels at the C2 shape come
+# from the FETCH_SIZE / WRITE_SIZE counter passes summarised in this file (bench.py cannot run the profiler
+# itself).  The summary is stamped with a hash of the kernel sources it was taken with; when the sources
+# have changed since, `traffic` is reported as null instead of a stale figure.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "gemm_kernels_c2_bf16.md")
+KERNEL_SOURCES = ("fsw_common.hpp", "fsw_gemm.hpp", "fsw_tiled.hip")
+
+
+def kernel_source_hash():
+    import hashlib
+
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "fusedswiglu_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def load_profiled_traffic(path=TRAFFIC_PROFILE):
+    """({kernel: HBM bytes per launch}, source hash the profile was taken with) parsed from the table
+    `| kernel | FETCH_SIZE KiB | WRITE_SIZE KiB | fetch scale | write scale |` of the profile summary."""
+    import re
+
+    traffic, stamp = {}, None
+    try:
+        text = open(path).read()
+    except OSError:
+        return traffic, stamp
+    for m in re.finditer(r"^\|\s*(\w+_dual_gemm)\s*\|\s*(\d+)\s*\|\s*(\d+)\s*\|\s*([\d.]+)\s*\|\s*([\d.]+)\s*\|", text, flags=re.M):
+        name, fetch, write, fs, ws = m.group(1), int(m.group(2)), int(m.group(3)), float(m.group(4)), float(m.group(5))
+        traffic[name] = int((fetch * fs + write * ws) * 1024)
+    m = re.search(r"kernel-source-sha256:\s*([0-9a-f]{16})", text)
+    if m:
+        stamp = m.group(1)
+    return traffic, stamp
 
 
 def parse():
@@ -62,11 +88,76 @@ def gpu_time_ms(fn, iters, warmup=3):
     return e0.elapsed_time(e1) / iters
 
 
+def other_configs(dev, c2_tensors):
+    """Event-timed fwd+bwd steps beside the headline: C3 (fp16, ragged I) and C5 (bf16, large) fused and
+    eager, the eager step and the memory-saving (recompute) step at C2, and single vendor GEMMs of the
+    three operand layouts at the C2 shape.  TFLOP/s by the same convention (12*T*D*I per step)."""
+    import torch
+    import torch.nn.functional as F
+
+    from fusedswiglu_amd import FastAccumFusedSwiGLU, FusedSwiGLU
+    from fusedswiglu_amd.ops import swiglu
+
+    def fused_step(fn, x, wg, wu, dout):
+        def run():
+            x.grad = wg.grad = wu.grad = None
+            fn(x, wg, wu).backward(dout)
+        return run
+
+    def eager_step(x, wg, wu, dout):
+        def run():
+            x.grad = wg.grad = wu.grad = None
+            (F.silu(x @ wg) * (x @ wu)).backward(dout)
+        return run
+
+    def rec(ms, flop):
+        return {"ms": round(ms, 4), "tflops": round(flop / ms / 1e9, 1)}
+
+    out = {}
+    x, wg, wu, dout = c2_tensors
+    T, D, I = x.shape[0] * x.shape[1], x.shape[2], wg.shape[1]
+    flop = 12.0 * T * D * I
+    out["C2_bf16"] = {
+        "shape": "x [4,2048,4096], W [4096,12288]",
+        "fused": rec(gpu_time_ms(fused_step(FusedSwiGLU.apply, x, wg, wu, dout), iters=10), flop),
+        "fused_recompute": rec(gpu_time_ms(fused_step(lambda a, b, c: swiglu(a, b, c, recompute=True), x, wg, wu, dout), iters=10), flop),
+        "eager_pytorch": rec(gpu_time_ms(eager_step(x, wg, wu, dout), iters=10), flop),
+    }
+    # single vendor GEMMs (torch.matmul -> hipBLASLt/rocBLAS) of the three layouts, 2*T*D*I flop each
+    xd, wd = x.detach().reshape(T, D), wg.detach()
+    dg = dout.reshape(T, I)
+    gflop = 2.0 * T * D * I
+    out["C2_bf16"]["vendor_gemm"] = {
+        "NN_forward_like": rec(gpu_time_ms(lambda: torch.matmul(xd, wd), iters=10), gflop),
+        "NT_input_grad_like": rec(gpu_time_ms(lambda: torch.matmul(dg, wd.t()), iters=10), gflop),
+        "TN_weight_grad_like": rec(gpu_time_ms(lambda: torch.matmul(xd.t(), dg), iters=10), gflop),
+    }
+    for name, fn, dt, xs, I2, iters in (("C3_fp16", FastAccumFusedSwiGLU.apply, torch.float16, (2, 4096, 4096), 11008, 10),
+                                        ("C5_bf16", FusedSwiGLU.apply, torch.bfloat16, (8, 4096, 8192), 28672, 3)):
+        torch.manual_seed(1)
+        D2 = xs[-1]
+        x2 = torch.randn(*xs, device=dev, dtype=torch.float32).to(dt).requires_grad_(True)
+        wg2 = (torch.randn(D2, I2, device=dev, dtype=torch.float32) / D2 ** 0.5).to(dt).requires_grad_(True)
+        wu2 = (torch.randn(D2, I2, device=dev, dtype=torch.float32) / D2 ** 0.5).to(dt).requires_grad_(True)
+        dy2 = torch.randn(*xs[:-1], I2, device=dev, dtype=torch.float32).to(dt)
+        fl2 = 12.0 * xs[0] * xs[1] * D2 * I2
+        out[name] = {
+            "shape": f"x {list(xs)}, W [{D2},{I2}]",
+            "fused": rec(gpu_time_ms(fused_step(fn, x2, wg2, wu2, dy2), iters=iters, warmup=2), fl2),
+            "eager_pytorch": rec(gpu_time_ms(eager_step(x2, wg2, wu2, dy2), iters=iters, warmup=2), fl2),
+        }
+        out[name]["fused_over_eager"] = round(out[name]["eager_pytorch"]["ms"] / out[name]["fused"]["ms"], 3)
+        del x2, wg2, wu2, dy2
+        torch.cuda.empty_cache()
+    out["C2_bf16"]["fused_over_eager"] = round(out["C2_bf16"]["eager_pytorch"]["ms"] / out["C2_bf16"]["fused"]["ms"], 3)
+    return out
+
+
 def main():
     args = parse()
     if args.gpus != 1:
-        print("bench.py: this build runs on ONE GPU; --gpus must be 1 (multi-GPU sharding is "
-              "described in DESIGN.md, not implemented)", file=sys.stderr)
+        print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no collective, sharding or rank code "
+              "is part of it, so there is no figure at several GPUs to report)", file=sys.stderr)
         sys.exit(2)
 
     import torch
@@ -128,6 +219,7 @@ def main():
             rec["gbs"] = round(10.0 * T * I / ms / 1e6, 1)  # 3 reads + 2 writes of 2 bytes per element
             rec["frac_hbm_peak"] = round(rec["gbs"] / PEAK_HBM_GBS, 4)
         kernels[name] = rec
+    profiled, stamp = load_profiled_traffic()
     gemm_names = [k for k in kernels if "tflops" in kernels[k]]
     dominant = max(gemm_names, key=lambda k: kernels[k]["ms"])
     achieved = 4.0 * T * D * I / kernels[dominant]["ms"] / 1e9
@@ -138,9 +230,11 @@ def main():
         "peak": PEAK_BF16_TFLOPS,
         "unit": "TFLOP/s",
         "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
-        "traffic": PROFILED_TRAFFIC_BYTES.get(dominant),
+        "traffic": profiled.get(dominant) if stamp == kernel_source_hash() else None,
         "algorithmic_flop_per_launch": 4.0 * T * D * I,
     }
+    if roofline["traffic"] is None:
+        roofline["traffic_note"] = "no counter profile of the current kernel sources in profiles/gemm_kernels_c2_bf16.md"
 
     result = {
         "metric": "fwd+bwd TFLOP/s & % bf16 MFMA peak, 8192 tok, d=4096->12288",
@@ -170,19 +264,19 @@ def main():
         ceil = {}
         for name, rnd in (("mfma_constant_operands_tflops", 0), ("mfma_normal_operands_tflops", 1)):
             fl = ctypes.c_double(0.0)
-            run = lambda: _abi.check(L.fsw_probe_mfma(rnd, 20000, ncu, p(sink), stream, ctypes.byref(fl)))  # noqa: E731
+            run = lambda: _abi.check(_abi.bench_lib().fsw_probe_mfma(rnd, 20000, ncu, p(sink), stream, ctypes.byref(fl)))  # noqa: E731
             ms = gpu_time_ms(run, iters=3, warmup=1)
             ceil[name] = round(fl.value / ms / 1e9, 1)
-        # the matrix cores beside the tiled kernels' own data movement (reads from LDS, L2-hit loads into LDS)
+        # the 16x16x32 instruction the tiled kernels use (mix 0 of the probe: no data movement beside it)
         window = torch.empty(8 << 20, device=dev, dtype=torch.uint8).fill_(60)
-        for name, mix in (("mfma_16x16x32_normal_operands_tflops", 0), ("mfma_with_kernel_data_movement_tflops", 1)):
+        for name, mix in (("mfma_16x16x32_normal_operands_tflops", 0),):
             fl = ctypes.c_double(0.0)
-            run = lambda: _abi.check(L.fsw_probe_mfma_mix(mix, 10000, 2 * ncu, p(window), window.numel(), p(sink), stream, ctypes.byref(fl)))  # noqa: E731
+            run = lambda: _abi.check(_abi.bench_lib().fsw_probe_mfma_mix(mix, 10000, 2 * ncu, p(window), window.numel(), p(sink), stream, ctypes.byref(fl)))  # noqa: E731
             ms = gpu_time_ms(run, iters=3, warmup=1)
             ceil[name] = round(fl.value / ms / 1e9, 1)
         del window
         big = torch.empty(1 << 31, device=dev, dtype=torch.uint8).fill_(1)
-        ms = gpu_time_ms(lambda: _abi.check(L.fsw_probe_stream_read(p(big), big.numel(), p(sink), stream)), iters=5, warmup=2)
+        ms = gpu_time_ms(lambda: _abi.check(_abi.bench_lib().fsw_probe_stream_read(p(big), big.numel(), p(sink), stream)), iters=5, warmup=2)
         ceil["hbm_stream_read_gbs"] = round(big.numel() / ms / 1e6, 1)
         del big
         result["measured_ceilings"] = ceil
@@ -195,9 +289,13 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    # ---- skinny-M forward (weight streaming, HBM bound), forward only, no pre-activation stores
+    # ---- the other configurations, the eager PyTorch step and the vendor GEMMs on the same box
     if not args.no_extra:
         del out, g, u, dG, dU, dx, dWg, dWu
+        result["other_configs"] = other_configs(dev, (x, wg, wu, dout))
+
+    # ---- skinny-M forward (weight streaming, HBM bound), forward only, no pre-activation stores
+    if not args.no_extra:
         D4, I4 = 8192, 28672
         w_sets = [((torch.randn(D4, I4, device=dev, dtype=dt) / D4 ** 0.5), (torch.randn(D4, I4, device=dev, dtype=dt) / D4 ** 0.5))
                   for _ in range(2)]

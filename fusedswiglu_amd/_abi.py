@@ -13,6 +13,8 @@ import threading
 
 _CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIBRARY_PATH = os.path.join(_CSRC, "libfusedswiglu.so")
+#: machine probes for the benchmark harness: a separate library, not part of the drop-in boundary
+BENCH_LIBRARY_PATH = os.path.join(_CSRC, "libfusedswiglu_bench.so")
 
 DTYPE_BF16 = 0
 DTYPE_FP16 = 1
@@ -29,7 +31,6 @@ EXPORTED_SYMBOLS = (
     "fsw_status_string",
     "fsw_last_error",
     "fsw_uses_tiled_kernel",
-    "fsw_force_edge_kernels",
     "fsw_workspace_bytes",
     "fsw_swiglu_forward",
     "fsw_elementwise_backward",
@@ -37,10 +38,9 @@ EXPORTED_SYMBOLS = (
     "fsw_input_grad",
     "fsw_input_grad_noalloc",
     "fsw_weight_grad",
-    "fsw_probe_mfma",
-    "fsw_probe_stream_read",
-    "fsw_probe_mfma_mix",
 )
+#: every symbol include/fusedswiglu_bench.h declares (libfusedswiglu_bench.so)
+BENCH_SYMBOLS = ("fsw_probe_mfma", "fsw_probe_stream_read", "fsw_probe_mfma_mix")
 
 
 class FusedSwiGLUError(RuntimeError):
@@ -62,7 +62,7 @@ _lock = threading.Lock()
 def build_library(verbose: bool = False, jobs: int = 4) -> str:
     """Compile the HIP sources for gfx950 with hipcc (works without a GPU) and return the
     path of the shared library.  Always recompiles."""
-    global _lib
+    global _lib, _bench_lib
     cmd = ["make", "-C", _CSRC, f"-j{jobs}", "-B"]
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if verbose or res.returncode != 0:
@@ -70,6 +70,7 @@ def build_library(verbose: bool = False, jobs: int = 4) -> str:
     if res.returncode != 0:
         raise RuntimeError("building libfusedswiglu.so failed")
     _lib = None
+    _bench_lib = None
     return LIBRARY_PATH
 
 
@@ -96,8 +97,6 @@ def lib() -> ctypes.CDLL:
         L.fsw_last_error.argtypes = []
         L.fsw_uses_tiled_kernel.restype = ci
         L.fsw_uses_tiled_kernel.argtypes = [ci, i64, i64, i64, i64, i64, i64, i64, ctypes.c_uint]
-        L.fsw_force_edge_kernels.restype = None
-        L.fsw_force_edge_kernels.argtypes = [ci]
         L.fsw_swiglu_forward.restype = ci
         L.fsw_swiglu_forward.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, vp]
         L.fsw_elementwise_backward.restype = ci
@@ -112,14 +111,32 @@ def lib() -> ctypes.CDLL:
         L.fsw_weight_grad.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, i64, ci, vp]
         L.fsw_workspace_bytes.restype = i64
         L.fsw_workspace_bytes.argtypes = [ci, i64, i64, i64]
-        L.fsw_probe_mfma.restype = ci
-        L.fsw_probe_mfma.argtypes = [ci, ci, ci, vp, vp, ctypes.POINTER(ctypes.c_double)]
-        L.fsw_probe_stream_read.restype = ci
-        L.fsw_probe_stream_read.argtypes = [vp, i64, vp, vp]
-        L.fsw_probe_mfma_mix.restype = ci
-        L.fsw_probe_mfma_mix.argtypes = [ci, ci, ci, vp, i64, vp, vp, ctypes.POINTER(ctypes.c_double)]
         _lib = L
     return _lib
+
+
+_bench_lib = None
+
+
+def bench_lib() -> ctypes.CDLL:
+    """The probe library of the benchmark harness (include/fusedswiglu_bench.h)."""
+    global _bench_lib
+    if _bench_lib is not None:
+        return _bench_lib
+    with _lock:
+        if _bench_lib is None:
+            if not os.path.exists(BENCH_LIBRARY_PATH):
+                raise LibraryNotBuiltError(f"{BENCH_LIBRARY_PATH} not found; build it with `make -C {_CSRC}`")
+            L = ctypes.CDLL(BENCH_LIBRARY_PATH)
+            vp, i64, ci = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+            L.fsw_probe_mfma.restype = ci
+            L.fsw_probe_mfma.argtypes = [ci, ci, ci, vp, vp, ctypes.POINTER(ctypes.c_double)]
+            L.fsw_probe_stream_read.restype = ci
+            L.fsw_probe_stream_read.argtypes = [vp, i64, vp, vp]
+            L.fsw_probe_mfma_mix.restype = ci
+            L.fsw_probe_mfma_mix.argtypes = [ci, ci, ci, vp, i64, vp, vp, ctypes.POINTER(ctypes.c_double)]
+            _bench_lib = L
+    return _bench_lib
 
 
 def check(status: int) -> None:

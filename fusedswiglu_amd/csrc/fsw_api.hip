@@ -1,7 +1,6 @@
 // extern "C" entry points of libfusedswiglu: argument validation, kernel selection, status codes.
 #include "../../include/fusedswiglu.h"
 #include "fsw_internal.hpp"
-#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <mutex>
@@ -9,7 +8,6 @@
 namespace {
 
 thread_local char g_err[512] = "";
-std::atomic<int> g_force_edge{0};
 
 int fail(int code, const char* fmt, ...) {
   va_list ap;
@@ -66,11 +64,8 @@ const char* fsw_status_string(int status) {
 
 const char* fsw_last_error(void) { return g_err; }
 
-void fsw_force_edge_kernels(int on) { g_force_edge.store(on ? 1 : 0); }
-
 int fsw_uses_tiled_kernel(int step, int64_t T, int64_t D, int64_t I, int64_t ldx, int64_t ldw,
                           int64_t ldo, int64_t ld_grad, unsigned pointer_alignment) {
-  if (g_force_edge.load()) return 0;
   // stand-in pointers that carry only the alignment
   const void* ptr = (const void*)(uintptr_t)(pointer_alignment ? pointer_alignment : 1);
   fsw::Problem p{};
@@ -78,7 +73,7 @@ int fsw_uses_tiled_kernel(int step, int64_t T, int64_t D, int64_t I, int64_t ldx
   p.out = p.g = p.u = p.dx = p.dWg = p.dWu = (void*)ptr;
   p.T = T; p.D = D; p.I = I; p.ldx = ldx; p.ldw = ldw; p.ldo = ldo; p.lddx = ld_grad; p.lddw = ld_grad;
   switch (step) {
-    case 0:
+    case 0: return fsw::skinny_forward_ok(p) ? 2 : (fsw::fast_path_ok_forward(p) ? 1 : 0);
     case 3: return fsw::fast_path_ok_forward(p) ? 1 : 0;
     case 1: return fsw::fast_path_ok_input_grad(p) ? 1 : 0;
     case 2: return fsw::fast_path_ok_weight_grad(p) ? 1 : 0;
@@ -109,8 +104,8 @@ int fsw_swiglu_forward(const void* x, const void* w_gate, const void* w_up, void
   p.x = x; p.wg = w_gate; p.wu = w_up; p.out = out; p.g = xw_gate; p.u = xw_up;
   p.T = T; p.D = D; p.I = I; p.ldx = ldx; p.ldw = ldw; p.ldo = ldo;
   hipStream_t s = (hipStream_t)stream;
-  if (!g_force_edge.load() && fsw::skinny_forward_ok(p)) return launched(fn, fsw::launch_forward_skinny(dtype, p, s));
-  if (!g_force_edge.load() && fsw::fast_path_ok_forward(p)) return launched(fn, fsw::launch_forward_fast(dtype, p, s));
+  if (fsw::skinny_forward_ok(p)) return launched(fn, fsw::launch_forward_skinny(dtype, p, s));
+  if (fsw::fast_path_ok_forward(p)) return launched(fn, fsw::launch_forward_fast(dtype, p, s));
   return launched(fn, fsw::launch_forward_generic(dtype, p, s));
 }
 
@@ -132,7 +127,7 @@ int fsw_gating_grad_recompute(const void* x, const void* w_gate, const void* w_u
   p.x = x; p.wg = w_gate; p.wu = w_up; p.dout = grad_out; p.g = grad_xw_gate; p.u = grad_xw_up;
   p.T = T; p.D = D; p.I = I; p.ldx = ldx; p.ldw = ldw; p.ldo = ldo;
   hipStream_t s = (hipStream_t)stream;
-  if (!g_force_edge.load() && fsw::fast_path_ok_forward(p)) return launched(fn, fsw::launch_forward_fast(dtype, p, s));
+  if (fsw::fast_path_ok_forward(p)) return launched(fn, fsw::launch_forward_fast(dtype, p, s));
   return launched(fn, fsw::launch_forward_generic(dtype, p, s));
 }
 
@@ -173,7 +168,7 @@ static int input_grad_checked(const char* fn, const void* grad_xw_gate, const vo
   p.dG = grad_xw_gate; p.dU = grad_xw_up; p.wg = w_gate; p.wu = w_up; p.dx = grad_x;
   p.T = T; p.D = D; p.I = I; p.ldo = ldo; p.ldw = ldw; p.lddx = ld_dx;
   hipStream_t s = (hipStream_t)stream;
-  if (!g_force_edge.load() && fsw::fast_path_ok_input_grad(p)) {
+  if (fsw::fast_path_ok_input_grad(p)) {
     const bool ws_ok = workspace && workspace_bytes > 0 && ((uintptr_t)workspace & 15) == 0;
     return launched(fn, fsw::launch_input_grad_fast(dtype, p, s, ws_ok ? workspace : nullptr, ws_ok ? workspace_bytes : 0));
   }
@@ -209,12 +204,14 @@ int fsw_weight_grad(const void* x, const void* grad_xw_up, const void* grad_xw_g
   p.x = x; p.dG = grad_xw_gate; p.dU = grad_xw_up; p.dWg = grad_w_gate; p.dWu = grad_w_up;
   p.T = T; p.D = D; p.I = I; p.ldx = ldx; p.ldo = ldo; p.lddw = ld_dw;
   hipStream_t s = (hipStream_t)stream;
-  if (!g_force_edge.load() && fsw::fast_path_ok_weight_grad(p)) {
+  if (fsw::fast_path_ok_weight_grad(p)) {
     const bool ws_ok = workspace && workspace_bytes > 0 && ((uintptr_t)workspace & 15) == 0;
     return launched(fn, fsw::launch_weight_grad_fast(dtype, p, s, ws_ok ? workspace : nullptr, ws_ok ? workspace_bytes : 0));
   }
   return launched(fn, fsw::launch_weight_grad_generic(dtype, p, s));
 }
+
+}  // extern "C"
 
 // ---- the entry point that allocates nothing -------------------------------------------------
 // Scratch for the split reduction of fsw_input_grad_noalloc: one copy per GPU, part of the library's
@@ -248,6 +245,8 @@ void* scratch_address(const char* fn) {
   return g_scratch_ptr[dev];
 }
 }  // namespace
+
+extern "C" {
 
 int fsw_input_grad_noalloc(const void* grad_xw_gate, const void* grad_xw_up, const void* w_gate,
                            const void* w_up, void* grad_x, int64_t T, int64_t D, int64_t I, int64_t ldo,

@@ -2,6 +2,7 @@
 // a register-only MFMA loop (no memory traffic at all) and a streaming read.  They only enqueue a
 // kernel; the caller times them with events on the same stream.
 #include "../../include/fusedswiglu.h"
+#include "../../include/fusedswiglu_bench.h"
 #include "fsw_common.hpp"
 
 namespace fsw {

@@ -110,7 +110,9 @@ __global__ __launch_bounds__(kSkThreads) void fsw_skinny_forward_kernel(GemmPara
       case 1: wait_vmcnt_and_barrier<1 * kPerStage>(); break;
       default: wait_vmcnt_and_barrier<0>(); break;
     }
-    // the barrier also says every wave has finished reading stage kt-1, which the next loads overwrite
+    // The barrier also says every wave has finished reading stage kt-1, which the next loads overwrite: each
+    // of those fragment reads feeds an MFMA the wave issued before it reached the barrier, and an MFMA is
+    // not issued before its operands have returned from LDS.
     issue(kt + kSkStages - 1);
     const FSW_LDS char* sa = smem_l + (kt % kSkStages) * kSkStage;
     const FSW_LDS char* sb = sa + kSkABytes;

@@ -8,22 +8,24 @@ static bool mult8(long long v) { return v > 0 && (v & 7) == 0; }
 static bool al16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 // a per-lane byte offset inside one tile (up to 256 rows) must stay below 2^31
 static bool ld_ok(long long ld) { return mult8(ld) && ld < (1LL << 21); }
+// leading dimension of a result: the kernels keep it in an int and index rows in 64 bits
+static bool ld_out_ok(long long ld) { return mult8(ld) && ld < (1LL << 31); }
 static bool dims_ok(const Problem& p) {
   return mult8(p.D) && mult8(p.I) && p.T > 0 && p.T < (1LL << 31) && p.D < (1LL << 31) &&
          p.I < (1LL << 31);
 }
 
 bool fast_path_ok_forward(const Problem& p) {
-  return dims_ok(p) && ld_ok(p.ldx) && ld_ok(p.ldw) && mult8(p.ldo) && al16(p.x) && al16(p.wg) &&
+  return dims_ok(p) && ld_ok(p.ldx) && ld_ok(p.ldw) && ld_out_ok(p.ldo) && al16(p.x) && al16(p.wg) &&
          al16(p.wu) && al16(p.out) && al16(p.g) && al16(p.u) && al16(p.dout);
 }
 bool fast_path_ok_input_grad(const Problem& p) {
-  return dims_ok(p) && ld_ok(p.ldo) && ld_ok(p.ldw) && mult8(p.lddx) && al16(p.dG) && al16(p.dU) &&
+  return dims_ok(p) && ld_ok(p.ldo) && ld_ok(p.ldw) && ld_out_ok(p.lddx) && al16(p.dG) && al16(p.dU) &&
          al16(p.wg) && al16(p.wu) && al16(p.dx);
 }
 bool fast_path_ok_weight_grad(const Problem& p) {
   // x and dG/dU are read with the token index outermost: T itself may be any positive count
-  return dims_ok(p) && ld_ok(p.ldx) && ld_ok(p.ldo) && mult8(p.lddw) && al16(p.x) && al16(p.dG) &&
+  return dims_ok(p) && ld_ok(p.ldx) && ld_ok(p.ldo) && ld_out_ok(p.lddw) && al16(p.x) && al16(p.dG) &&
          al16(p.dU) && al16(p.dWg) && al16(p.dWu);
 }
 

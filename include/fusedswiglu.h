@@ -19,7 +19,8 @@
  *     accumulated in fp32 on the MFMA units for both (CDNA4 has no fp16-accumulate mode,
  *     so the reference's fp16 "fast accumulation" maps to fp32 accumulation).
  *   - `stream` is a hipStream_t (NULL = the default stream).  Calls only enqueue work; they
- *     never synchronize.  The library is stateless and re-entrant.
+ *     never synchronize.  The library keeps no state between calls and is re-entrant (the one
+ *     exception, the built-in scratch of fsw_input_grad_noalloc, is described there).
  *   - Return value: FSW_OK or an FSW_ERR_* code; arguments are validated before anything is
  *     enqueued.  fsw_last_error() gives a thread-local message for the last failure.
  *   - Operands whose dimensions and leading dimensions are multiples of 8 elements and whose
@@ -30,6 +31,11 @@
 #define FUSEDSWIGLU_H_
 
 #include <stdint.h>
+
+/* Every entry point is exported with default visibility; the libraries hide everything else. */
+#ifndef FSW_API
+#define FSW_API __attribute__((visibility("default")))
+#endif
 
 #ifdef __cplusplus
 extern "C" {
@@ -51,18 +57,16 @@ enum {
 };
 
 /* Library version (FSW_VERSION it was built with). */
-int fsw_version(void);
+FSW_API int fsw_version(void);
 /* Static description of a status code. */
-const char* fsw_status_string(int status);
+FSW_API const char* fsw_status_string(int status);
 /* Message of the calling thread's most recent failed call ("" if none). */
-const char* fsw_last_error(void);
-/* 1 if the arguments of the named step would run on the tiled kernels, 0 if on the
- * edge-shape kernel.  step: 0 forward, 1 input_grad, 2 weight_grad, 3 gating_grad_recompute.
- * Pure host logic. */
-int fsw_uses_tiled_kernel(int step, int64_t T, int64_t D, int64_t I, int64_t ldx, int64_t ldw,
+FSW_API const char* fsw_last_error(void);
+/* Which kernel the arguments of the named step would run on: 1 the tiled MFMA kernels, 2 the
+ * weight-streaming forward (step 0 with at most 128 tokens), 0 the edge-shape kernel.
+ * step: 0 forward, 1 input_grad, 2 weight_grad, 3 gating_grad_recompute.  Pure host logic. */
+FSW_API int fsw_uses_tiled_kernel(int step, int64_t T, int64_t D, int64_t I, int64_t ldx, int64_t ldw,
                           int64_t ldo, int64_t ld_grad, unsigned pointer_alignment);
-/* Test hook: nonzero forces every later call of this process onto the edge-shape kernels. */
-void fsw_force_edge_kernels(int on);
 
 /*
  * Forward: g = x Wg, u = x Wu, out = silu(g) * u.
@@ -72,7 +76,7 @@ void fsw_force_edge_kernels(int on);
  * xw_gate and xw_up (the pre-activations the backward needs) may both be NULL, in which
  * case they are not written (inference).
  */
-int fsw_swiglu_forward(const void* x, const void* w_gate, const void* w_up, void* out,
+FSW_API int fsw_swiglu_forward(const void* x, const void* w_gate, const void* w_up, void* out,
                        void* xw_gate, void* xw_up, int64_t T, int64_t D, int64_t I, int64_t ldx,
                        int64_t ldw, int64_t ldo, int dtype, void* stream);
 
@@ -82,7 +86,7 @@ int fsw_swiglu_forward(const void* x, const void* w_gate, const void* w_up, void
  * Replaces elementwise_backward + kernel (kernels_bf16.py:236-255, :210-234).  All five
  * arrays are dense with `numel` elements.
  */
-int fsw_elementwise_backward(const void* grad_out, const void* xw_gate, const void* xw_up,
+FSW_API int fsw_elementwise_backward(const void* grad_out, const void* xw_gate, const void* xw_up,
                              void* grad_xw_up, void* grad_xw_gate, int64_t numel, int dtype,
                              void* stream);
 
@@ -94,7 +98,7 @@ int fsw_elementwise_backward(const void* grad_out, const void* xw_gate, const vo
  * elements per layer; the reference has no such mode.
  *   x [T,D] (ldx)   w_gate, w_up [D,I] (ldw)   grad_out, grad_xw_up, grad_xw_gate [T,I] (ldo)
  */
-int fsw_gating_grad_recompute(const void* x, const void* w_gate, const void* w_up,
+FSW_API int fsw_gating_grad_recompute(const void* x, const void* w_gate, const void* w_up,
                               const void* grad_out, void* grad_xw_up, void* grad_xw_gate, int64_t T,
                               int64_t D, int64_t I, int64_t ldx, int64_t ldw, int64_t ldo, int dtype,
                               void* stream);
@@ -105,16 +109,16 @@ int fsw_gating_grad_recompute(const void* x, const void* w_gate, const void* w_u
  * tiles to `workspace` (device memory owned by the caller, 16-byte aligned, contents irrelevant) and
  * a second kernel adds them in a fixed order.  fsw_workspace_bytes gives a sufficient size for
  * step 1 (input_grad) or 2 (weight_grad); with workspace == NULL or a smaller size the call still
- * works, just without (or with a smaller) split.  Large problems never touch the workspace.
+ * works, just without the split.  Large problems never touch the workspace.
  */
-int64_t fsw_workspace_bytes(int step, int64_t T, int64_t D, int64_t I);
+FSW_API int64_t fsw_workspace_bytes(int step, int64_t T, int64_t D, int64_t I);
 
 /*
  * Input gradient: grad_x = grad_xw_gate Wg^T + grad_xw_up Wu^T, one kernel, one accumulator.
  * Replaces the two torch matmuls and the add at fused_swiglu/swiglu.py:45.
  *   grad_xw_gate, grad_xw_up [T,I] (ldo)   w_gate, w_up [D,I] (ldw)   grad_x [T,D] (ld_dx)
  */
-int fsw_input_grad(const void* grad_xw_gate, const void* grad_xw_up, const void* w_gate,
+FSW_API int fsw_input_grad(const void* grad_xw_gate, const void* grad_xw_up, const void* w_gate,
                    const void* w_up, void* grad_x, int64_t T, int64_t D, int64_t I, int64_t ldo,
                    int64_t ldw, int64_t ld_dx, void* workspace, int64_t workspace_bytes, int dtype,
                    void* stream);
@@ -131,7 +135,7 @@ int fsw_input_grad(const void* grad_xw_gate, const void* grad_xw_up, const void*
  * on a device looks the buffer's address up; make that call outside graph capture.
  */
 #define FSW_NOALLOC_SCRATCH_BYTES (32u << 20)
-int fsw_input_grad_noalloc(const void* grad_xw_gate, const void* grad_xw_up, const void* w_gate,
+FSW_API int fsw_input_grad_noalloc(const void* grad_xw_gate, const void* grad_xw_up, const void* w_gate,
                            const void* w_up, void* grad_x, int64_t T, int64_t D, int64_t I, int64_t ldo,
                            int64_t ldw, int64_t ld_dx, int dtype, void* stream);
 
@@ -142,27 +146,10 @@ int fsw_input_grad_noalloc(const void* grad_xw_gate, const void* grad_xw_up, con
  *   x [T,D] (ldx)   grad_xw_up, grad_xw_gate [T,I] (ldo)   grad_w_up, grad_w_gate [D,I] (ld_dw)
  * Argument order (up before gate) follows fused_bmm.
  */
-int fsw_weight_grad(const void* x, const void* grad_xw_up, const void* grad_xw_gate,
+FSW_API int fsw_weight_grad(const void* x, const void* grad_xw_up, const void* grad_xw_gate,
                     void* grad_w_up, void* grad_w_gate, int64_t T, int64_t D, int64_t I,
                     int64_t ldx, int64_t ldo, int64_t ld_dw, void* workspace, int64_t workspace_bytes,
                     int dtype, void* stream);
-
-/*
- * Machine probes for the benchmark harness (no counterpart in the reference).  Each call enqueues one
- * kernel on `stream`; the caller times it with events.  sink4 is a 4-byte device scratch word.
- * fsw_probe_mfma: `workgroups` x 8 waves issue `iters` x 8 back-to-back 32x32x16 bf16 MFMAs from
- * registers (operands constant, or ~N(0,1) if random_operands != 0); *flop_out receives the flop count.
- * fsw_probe_stream_read: grid-stride 16-byte reads of `bytes` bytes at buf (16-byte aligned).
- * fsw_probe_mfma_mix: `workgroups` x 8 waves issue `iters` x 32 16x16x32 bf16 MFMAs on ~N(0,1) operands
- * with, per 8 MFMAs, the data movement of mix 0: none, 1: three 16-byte LDS reads per lane + one 1 KiB
- * direct global->LDS load per wave (what the tiled kernels do), 2: two reads + one load, 3: three reads,
- * 4: one load.  The loads walk `bytes` bytes at buf (a multiple of 256 KiB, >= 1 MiB, < 2 GiB).
- */
-int fsw_probe_mfma(int random_operands, int iters, int workgroups, void* sink4, void* stream,
-                   double* flop_out);
-int fsw_probe_stream_read(const void* buf, int64_t bytes, void* sink4, void* stream);
-int fsw_probe_mfma_mix(int mix, int iters, int workgroups, const void* buf, int64_t bytes, void* sink4,
-                       void* stream, double* flop_out);
 
 #ifdef __cplusplus
 }

@@ -21,15 +21,35 @@ def L():
     return _abi.lib()
 
 
-def test_header_symbols_all_exported(L):
-    header = open(os.path.join(ROOT, "include", "fusedswiglu.h")).read()
+def _declared(header_name):
+    header = open(os.path.join(ROOT, "include", header_name)).read()
     header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
-    declared = set(re.findall(r"\b(fsw_[a-z_0-9]+)\s*\(", header))
+    return set(re.findall(r"\b(fsw_[a-z_0-9]+)\s*\(", header))
+
+
+def _exported(path):
+    import subprocess
+
+    out = subprocess.run(["nm", "-D", "--defined-only", path], stdout=subprocess.PIPE, text=True, check=True).stdout
+    return {line.split()[-1] for line in out.splitlines() if " T " in line}
+
+
+def test_header_symbols_all_exported(L):
+    """The drop-in library exports exactly what include/fusedswiglu.h declares - the path and nothing else;
+    the benchmark probes live in a library and a header of their own."""
+    declared = _declared("fusedswiglu.h")
     assert declared == set(_abi.EXPORTED_SYMBOLS)
+    assert _exported(_abi.LIBRARY_PATH) == declared
     for name in declared:
         assert getattr(L, name) is not None
+    header = open(os.path.join(ROOT, "include", "fusedswiglu.h")).read()
     m = re.search(r"#define FSW_VERSION (\d+)", header)
     assert L.fsw_version() == int(m.group(1))
+    assert "probe" not in header and "force_edge" not in header
+    bench = _declared("fusedswiglu_bench.h")
+    assert bench == set(_abi.BENCH_SYMBOLS) == _exported(_abi.BENCH_LIBRARY_PATH)
+    for name in bench:
+        assert getattr(_abi.bench_lib(), name) is not None
 
 
 def test_status_strings(L):
@@ -96,7 +116,8 @@ def test_backward_validation(L):
     assert L.fsw_workspace_bytes(0, 8192, 256, 768) == 0 and L.fsw_workspace_bytes(1, 0, 1, 1) == 0
 
 
-def test_probe_validation(L):
+def test_probe_validation():
+    L = _abi.bench_lib()
     f = L.fsw_probe_mfma_mix
     flop = ctypes.c_double(0.0)
     assert f(1, 10, 256, None, 8 << 20, P, None, ctypes.byref(flop)) == 3          # no source window
@@ -122,12 +143,12 @@ def test_kernel_selection_logic(L):
     # the token count is free: it is never the contiguous index of an operand
     assert t(0, 8191, 4096, 12288, 4096, 12288, 12288, 12288, 16) == 1
     assert t(2, 8191, 4096, 12288, 4096, 12288, 12288, 12288, 16) == 1
-    L.fsw_force_edge_kernels(1)
-    try:
-        assert t(0, 8192, 4096, 12288, 4096, 12288, 12288, 12288, 16) == 0
-    finally:
-        L.fsw_force_edge_kernels(0)
-    assert t(0, 8192, 4096, 12288, 4096, 12288, 12288, 12288, 16) == 1
+    # few tokens: the forward streams the weights once with its own kernel (only the forward)
+    assert t(0, 128, 8192, 28672, 8192, 28672, 28672, 28672, 16) == 2 and t(0, 16, 8192, 28672, 8192, 28672, 28672, 28672, 16) == 2
+    assert t(0, 129, 8192, 28672, 8192, 28672, 28672, 28672, 16) == 1 and t(3, 16, 8192, 28672, 8192, 28672, 28672, 28672, 16) == 1
+    assert t(0, 16, 8192, 28672, 8192, 28672, 28672, 28672, 2) == 0
+    # result rows are indexed through a 32-bit leading dimension on the tiled kernels: beyond that, edge kernel
+    assert t(0, 8, 64, 64, 64, 64, 2 ** 31, 64, 16) == 0 and t(1, 512, 64, 64, 64, 64, 64, 2 ** 31 + 8, 16) == 0
 
 
 def test_python_boundary_errors_without_gpu():

@@ -330,16 +330,26 @@ def test_extreme_aspect_ratios(oracle, shape):
 
 
 # ---- boundary behaviour ---------------------------------------------------------------------------
+def _misaligned(t):
+    """The same values in storage that starts 2 bytes off a 16-byte boundary: such operands take the
+    edge-shape kernels (the tiled ones need 16-byte aligned pointers)."""
+    buf = torch.empty(t.numel() + 8, dtype=t.dtype, device=t.device)
+    view = buf[1:1 + t.numel()].view(t.shape)
+    view.copy_(t)
+    assert view.data_ptr() % 16 == 2 and view.is_contiguous()
+    return view
+
+
 def test_edge_kernels_agree_with_tiled_kernels(oracle):
-    """Force the edge-shape kernels onto an aligned problem: both paths meet the oracle."""
+    """An aligned problem on the tiled kernels and, from misaligned copies of the same operands, on the
+    edge-shape kernels: both paths meet the oracle and each other."""
     dtype, shape = torch.bfloat16, (2, 136, 264, 520)
+    B, S, D, I = shape
     (x, wg, wu, dy), (tx, twg, twu, tdy) = make(oracle, shape, dtype, seed=7)
+    assert _abi.lib().fsw_uses_tiled_kernel(0, B * S, D, I, D, I, I, I, 16) == 1
+    assert _abi.lib().fsw_uses_tiled_kernel(0, B * S, D, I, D, I, I, I, 2) == 0
     tiled = run_fwd_bwd(dtype, tx, twg, twu, tdy)
-    _abi.lib().fsw_force_edge_kernels(1)
-    try:
-        edge = run_fwd_bwd(dtype, tx, twg, twu, tdy)
-    finally:
-        _abi.lib().fsw_force_edge_kernels(0)
+    edge = run_fwd_bwd(dtype, _misaligned(tx), _misaligned(twg), _misaligned(twu), _misaligned(tdy))
     exact = (oracle.fused_swiglu_fwd(x, wg, wu)[0],) + oracle.swiglu_backward(x, wg, wu, dy)
     for a, b, e in zip(tiled, edge, exact):
         assert oracle.rel_error(np64(a), e) < TOL[dtype] and oracle.rel_error(np64(b), e) < TOL[dtype]
