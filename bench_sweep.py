@@ -5,9 +5,11 @@ The reference's README (README.md:41-63) plots TFLOP/s for batch 4, sequence 204
 d_intermediate = 3 * d_model, d_model = 256 ... 4096, forward and forward+backward, bf16 and fp16,
 for its fused kernels against eager PyTorch.  This script measures the same grid for this library
 and for eager PyTorch (rocBLAS/hipBLASLt matmuls + elementwise kernels) on the same box and prints
-a markdown table.  Flop convention: forward 4*T*D*I, forward+backward 12*T*D*I.
+a markdown table; with --out it also writes the table, the raw numbers (JSON) and the four plots of
+the README (bf16 / fp16 x forward / forward+backward, fused against eager) into that directory.
+Flop convention: forward 4*T*D*I, forward+backward 12*T*D*I.
 
-    python bench_sweep.py [--step 512] [--iters 10]
+    python bench_sweep.py [--step 128] [--iters 10] [--out DIR]
 """
 import argparse
 import sys
@@ -38,8 +40,9 @@ def time_ms(fn, iters, warmup=3, min_ms=40.0):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--step", type=int, default=512)
+    ap.add_argument("--step", type=int, default=128, help="d_model step; 128 is the README's grid")
     ap.add_argument("--iters", type=int, default=10)
+    ap.add_argument("--out", default=None, help="directory for sweep.md, sweep.json and the four PNG plots")
     args = ap.parse_args()
     import torch
 
@@ -48,10 +51,12 @@ def main():
     dev = "cuda:0"
     B, S = 4, 2048
     T = B * S
-    print("| dtype | d_model | fused fwd TFLOP/s | eager fwd | fused fwd+bwd TFLOP/s | eager fwd+bwd |")
-    print("|---|---|---|---|---|---|")
+    lines = ["| dtype | d_model | fused fwd TFLOP/s | eager fwd | fused fwd+bwd TFLOP/s | eager fwd+bwd |",
+             "|---|---|---|---|---|---|"]
+    print("\n".join(lines))
+    rows = []
     for dtype, fn in ((torch.bfloat16, FusedSwiGLU), (torch.float16, FastAccumFusedSwiGLU)):
-        for D in [256] + list(range(args.step, 4097, args.step)):
+        for D in sorted(set([256] + list(range(256, 4097, args.step)) + [4096])):
             I = 3 * D
             torch.manual_seed(0)
             x = torch.randn(B, S, D, device=dev, dtype=dtype, requires_grad=True)
@@ -78,7 +83,45 @@ def main():
             f = 4.0 * T * D * I
             r = [f / time_ms(fused_fwd, args.iters) / 1e9, f / time_ms(eager_fwd, args.iters) / 1e9,
                  3 * f / time_ms(fused_fb, args.iters) / 1e9, 3 * f / time_ms(eager_fb, args.iters) / 1e9]
-            print(f"| {'bf16' if dtype == torch.bfloat16 else 'fp16'} | {D} | {r[0]:.0f} | {r[1]:.0f} | {r[2]:.0f} | {r[3]:.0f} |", flush=True)
+            name = "bf16" if dtype == torch.bfloat16 else "fp16"
+            lines.append(f"| {name} | {D} | {r[0]:.0f} | {r[1]:.0f} | {r[2]:.0f} | {r[3]:.0f} |")
+            print(lines[-1], flush=True)
+            rows.append({"dtype": name, "d_model": D, "fused_fwd": r[0], "eager_fwd": r[1], "fused_fwd_bwd": r[2], "eager_fwd_bwd": r[3]})
+    if args.out:
+        write_outputs(args.out, lines, rows, args.step)
+
+
+def write_outputs(out_dir, lines, rows, step):
+    import json
+
+    import matplotlib
+
+    matplotlib.use("Agg")
+    import matplotlib.pyplot as plt
+
+    os.makedirs(out_dir, exist_ok=True)
+    head = (f"Sweep on the reference's published protocol (batch 4, sequence 2048, d_intermediate = 3 * d_model, "
+            f"d_model 256 ... 4096 step {step}), one MI355X, `python bench_sweep.py --step {step} --out DIR`; "
+            "TFLOP/s, fused = this library, eager = PyTorch matmuls + elementwise kernels on the same box.\n\n")
+    with open(os.path.join(out_dir, "sweep.md"), "w") as f:
+        f.write(head + "\n".join(lines) + "\n")
+    with open(os.path.join(out_dir, "sweep.json"), "w") as f:
+        json.dump(rows, f, indent=0)
+    for name in ("bf16", "fp16"):
+        sel = [r for r in rows if r["dtype"] == name]
+        xs = [r["d_model"] for r in sel]
+        for key, title in (("fwd", "forward"), ("fwd_bwd", "forward + backward")):
+            plt.figure(figsize=(7, 4.2))
+            plt.plot(xs, [r["fused_" + key] for r in sel], "o-", ms=3, label="fused (this library, MI355X)")
+            plt.plot(xs, [r["eager_" + key] for r in sel], "s--", ms=3, label="eager PyTorch (rocBLAS/hipBLASLt)")
+            plt.xlabel("d_model (batch 4, sequence 2048, d_intermediate = 3 d_model)")
+            plt.ylabel("TFLOP/s")
+            plt.title(f"SwiGLU {title}, {name}")
+            plt.grid(alpha=0.3)
+            plt.legend()
+            plt.tight_layout()
+            plt.savefig(os.path.join(out_dir, f"{name}_{key}.png"), dpi=110)
+            plt.close()
 
 
 if __name__ == "__main__":
