@@ -124,9 +124,11 @@ def test_autocast_casts_like_the_reference_functions(oracle):
         m(tx.float())
 
 
-def test_torch_compile_keeps_the_operator_opaque(oracle):
-    """torch.compile (aot_eager backend: no code generation) traces through module and operator in
-    one graph and reproduces the eager results and gradients exactly."""
+@pytest.mark.parametrize("backend", ["aot_eager", "inductor"])
+def test_torch_compile_keeps_the_operator_opaque(oracle, backend):
+    """torch.compile traces through module and operator in one graph and reproduces the eager results and
+    gradients exactly: with the aot_eager backend (no code generation) and with the default inductor
+    backend, which has to treat the registered operators as opaque calls around its own generated code."""
     dtype, shape = torch.bfloat16, (2, 64, 128, 264)
     _, (tx, twg, twu, tdy) = inputs(oracle, shape, dtype, seed=16)
     m = fsw.SwiGLU(shape[2], shape[3], device=DEV)
@@ -138,7 +140,8 @@ def test_torch_compile_keeps_the_operator_opaque(oracle):
     oe.backward(tdy)
     ge = [xe.grad.clone(), m.w_gate.grad.clone(), m.w_up.grad.clone()]
     m.zero_grad(set_to_none=True)
-    cm = torch.compile(m, backend="aot_eager", fullgraph=True)
+    torch._dynamo.reset()
+    cm = torch.compile(m, backend=backend, fullgraph=True)
     xc = tx.clone().requires_grad_(True)
     oc = cm(xc)
     oc.backward(tdy)
