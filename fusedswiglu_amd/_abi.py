@@ -18,6 +18,9 @@ BENCH_LIBRARY_PATH = os.path.join(_CSRC, "libfusedswiglu_bench.so")
 
 DTYPE_BF16 = 0
 DTYPE_FP16 = 1
+#: OR-ed into a dtype code (or a workspace step): weights are stored "out x in" like nn.Linear.weight
+WEIGHTS_OUT_IN = 0x100
+STEP_DOWN_FORWARD, STEP_DOWN_INPUT_GRAD, STEP_DOWN_WEIGHT_GRAD = 4, 5, 6
 
 STEP_FORWARD, STEP_INPUT_GRAD, STEP_WEIGHT_GRAD = 0, 1, 2
 
@@ -38,6 +41,9 @@ EXPORTED_SYMBOLS = (
     "fsw_input_grad",
     "fsw_input_grad_noalloc",
     "fsw_weight_grad",
+    "fsw_down_proj_forward",
+    "fsw_down_proj_input_grad",
+    "fsw_down_proj_weight_grad",
 )
 #: every symbol include/fusedswiglu_bench.h declares (libfusedswiglu_bench.so)
 BENCH_SYMBOLS = ("fsw_probe_mfma", "fsw_probe_stream_read", "fsw_probe_mfma_mix")
@@ -109,6 +115,9 @@ def lib() -> ctypes.CDLL:
         L.fsw_input_grad_noalloc.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, vp]
         L.fsw_weight_grad.restype = ci
         L.fsw_weight_grad.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, i64, ci, vp]
+        for name in ("fsw_down_proj_forward", "fsw_down_proj_input_grad", "fsw_down_proj_weight_grad"):
+            getattr(L, name).restype = ci
+            getattr(L, name).argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, i64, ci, vp]
         L.fsw_workspace_bytes.restype = i64
         L.fsw_workspace_bytes.argtypes = [ci, i64, i64, i64]
         _lib = L

@@ -17,7 +17,13 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
-bool dtype_ok(int d) { return d == FSW_DTYPE_BF16 || d == FSW_DTYPE_FP16; }
+// `dtype` arguments carry the element type in the low byte and optional FSW_* layout flags above it
+bool dtype_ok(int d) {
+  const int e = d & 0xff;
+  return (e == FSW_DTYPE_BF16 || e == FSW_DTYPE_FP16) && (d & ~(0xff | FSW_WEIGHTS_OUT_IN)) == 0;
+}
+int elem_of(int d) { return d & 0xff; }
+bool out_in_of(int d) { return (d & FSW_WEIGHTS_OUT_IN) != 0; }
 bool al2(const void* p) { return ((uintptr_t)p & 1) == 0; }
 
 int check_dims(const char* fn, int64_t T, int64_t D, int64_t I) {
@@ -72,7 +78,8 @@ int fsw_uses_tiled_kernel(int step, int64_t T, int64_t D, int64_t I, int64_t ldx
   p.x = p.wg = p.wu = p.dG = p.dU = ptr;
   p.out = p.g = p.u = p.dx = p.dWg = p.dWu = (void*)ptr;
   p.T = T; p.D = D; p.I = I; p.ldx = ldx; p.ldw = ldw; p.ldo = ldo; p.lddx = ld_grad; p.lddw = ld_grad;
-  switch (step) {
+  p.w_out_in = (step & FSW_WEIGHTS_OUT_IN) != 0;
+  switch (step & 0xff) {
     case 0: return fsw::skinny_forward_ok(p) ? 2 : (fsw::fast_path_ok_forward(p) ? 1 : 0);
     case 3: return fsw::fast_path_ok_forward(p) ? 1 : 0;
     case 1: return fsw::fast_path_ok_input_grad(p) ? 1 : 0;
@@ -83,7 +90,16 @@ int fsw_uses_tiled_kernel(int step, int64_t T, int64_t D, int64_t I, int64_t ldx
 
 int64_t fsw_workspace_bytes(int step, int64_t T, int64_t D, int64_t I) {
   if (T <= 0 || D <= 0 || I <= 0) return 0;
-  return fsw::splitk_workspace_bytes(step, T, D, I);
+  const bool oi = (step & FSW_WEIGHTS_OUT_IN) != 0;
+  switch (step & 0xff) {
+    case 1: return fsw::splitk_workspace_bytes(oi ? 4 : 1, T, D, I);
+    case 2: return fsw::splitk_workspace_bytes(oi ? 5 : 2, T, D, I);
+    // down projection: forward y [T,D] over I; input grad [T,I] over D; weight grad [I,D] ([D,I]) over T
+    case 4: return fsw::gemm_workspace_bytes(oi ? 1 : 0, T, D, I);
+    case 5: return fsw::gemm_workspace_bytes(oi ? 0 : 1, T, I, D);
+    case 6: return oi ? fsw::gemm_workspace_bytes(2, D, I, T) : fsw::gemm_workspace_bytes(2, I, D, T);
+    default: return 0;
+  }
 }
 
 int fsw_swiglu_forward(const void* x, const void* w_gate, const void* w_up, void* out,
@@ -95,14 +111,16 @@ int fsw_swiglu_forward(const void* x, const void* w_gate, const void* w_up, void
     return fail(FSW_ERR_NULL_POINTER, "%s: xw_gate and xw_up must both be given or both be null", fn);
   if (!dtype_ok(dtype)) return fail(FSW_ERR_BAD_DTYPE, "%s: dtype %d is neither bf16 (0) nor fp16 (1)", fn, dtype);
   if (int e = check_dims(fn, T, D, I)) return e;
+  const bool oi = out_in_of(dtype);
+  dtype = elem_of(dtype);
   if (int e = check_ld(fn, "ldx", ldx, D)) return e;
-  if (int e = check_ld(fn, "ldw", ldw, I)) return e;
+  if (int e = check_ld(fn, "ldw", ldw, oi ? D : I)) return e;
   if (int e = check_ld(fn, "ldo", ldo, I)) return e;
   if (!al2(x) || !al2(w_gate) || !al2(w_up) || !al2(out) || !al2(xw_gate) || !al2(xw_up))
     return fail(FSW_ERR_ALIGNMENT, "%s: pointers must be 2-byte aligned", fn);
   fsw::Problem p{};
   p.x = x; p.wg = w_gate; p.wu = w_up; p.out = out; p.g = xw_gate; p.u = xw_up;
-  p.T = T; p.D = D; p.I = I; p.ldx = ldx; p.ldw = ldw; p.ldo = ldo;
+  p.T = T; p.D = D; p.I = I; p.ldx = ldx; p.ldw = ldw; p.ldo = ldo; p.w_out_in = oi;
   hipStream_t s = (hipStream_t)stream;
   if (fsw::skinny_forward_ok(p)) return launched(fn, fsw::launch_forward_skinny(dtype, p, s));
   if (fsw::fast_path_ok_forward(p)) return launched(fn, fsw::launch_forward_fast(dtype, p, s));
@@ -118,14 +136,16 @@ int fsw_gating_grad_recompute(const void* x, const void* w_gate, const void* w_u
     return fail(FSW_ERR_NULL_POINTER, "%s: all six arrays must be non-null", fn);
   if (!dtype_ok(dtype)) return fail(FSW_ERR_BAD_DTYPE, "%s: dtype %d is neither bf16 (0) nor fp16 (1)", fn, dtype);
   if (int e = check_dims(fn, T, D, I)) return e;
+  const bool oi = out_in_of(dtype);
+  dtype = elem_of(dtype);
   if (int e = check_ld(fn, "ldx", ldx, D)) return e;
-  if (int e = check_ld(fn, "ldw", ldw, I)) return e;
+  if (int e = check_ld(fn, "ldw", ldw, oi ? D : I)) return e;
   if (int e = check_ld(fn, "ldo", ldo, I)) return e;
   if (!al2(x) || !al2(w_gate) || !al2(w_up) || !al2(grad_out) || !al2(grad_xw_up) || !al2(grad_xw_gate))
     return fail(FSW_ERR_ALIGNMENT, "%s: pointers must be 2-byte aligned", fn);
   fsw::Problem p{};
   p.x = x; p.wg = w_gate; p.wu = w_up; p.dout = grad_out; p.g = grad_xw_gate; p.u = grad_xw_up;
-  p.T = T; p.D = D; p.I = I; p.ldx = ldx; p.ldw = ldw; p.ldo = ldo;
+  p.T = T; p.D = D; p.I = I; p.ldx = ldx; p.ldw = ldw; p.ldo = ldo; p.w_out_in = oi;
   hipStream_t s = (hipStream_t)stream;
   if (fsw::fast_path_ok_forward(p)) return launched(fn, fsw::launch_forward_fast(dtype, p, s));
   return launched(fn, fsw::launch_forward_generic(dtype, p, s));
@@ -138,6 +158,7 @@ int fsw_elementwise_backward(const void* grad_out, const void* xw_gate, const vo
   if (!grad_out || !xw_gate || !xw_up || !grad_xw_up || !grad_xw_gate)
     return fail(FSW_ERR_NULL_POINTER, "%s: all five arrays must be non-null", fn);
   if (!dtype_ok(dtype)) return fail(FSW_ERR_BAD_DTYPE, "%s: dtype %d is neither bf16 (0) nor fp16 (1)", fn, dtype);
+  dtype = elem_of(dtype);
   if (numel <= 0) return fail(FSW_ERR_BAD_SHAPE, "%s: numel must be positive (got %lld)", fn, (long long)numel);
   if (!al2(grad_out) || !al2(xw_gate) || !al2(xw_up) || !al2(grad_xw_up) || !al2(grad_xw_gate))
     return fail(FSW_ERR_ALIGNMENT, "%s: pointers must be 2-byte aligned", fn);
@@ -153,7 +174,7 @@ static int check_input_grad_args(const char* fn, const void* grad_xw_gate, const
   if (!dtype_ok(dtype)) return fail(FSW_ERR_BAD_DTYPE, "%s: dtype %d is neither bf16 (0) nor fp16 (1)", fn, dtype);
   if (int e = check_dims(fn, T, D, I)) return e;
   if (int e = check_ld(fn, "ldo", ldo, I)) return e;
-  if (int e = check_ld(fn, "ldw", ldw, I)) return e;
+  if (int e = check_ld(fn, "ldw", ldw, out_in_of(dtype) ? D : I)) return e;
   if (int e = check_ld(fn, "ld_dx", ld_dx, D)) return e;
   if (!al2(grad_xw_gate) || !al2(grad_xw_up) || !al2(w_gate) || !al2(w_up) || !al2(grad_x))
     return fail(FSW_ERR_ALIGNMENT, "%s: pointers must be 2-byte aligned", fn);
@@ -166,7 +187,8 @@ static int input_grad_checked(const char* fn, const void* grad_xw_gate, const vo
                               int64_t workspace_bytes, int dtype, void* stream) {
   fsw::Problem p{};
   p.dG = grad_xw_gate; p.dU = grad_xw_up; p.wg = w_gate; p.wu = w_up; p.dx = grad_x;
-  p.T = T; p.D = D; p.I = I; p.ldo = ldo; p.ldw = ldw; p.lddx = ld_dx;
+  p.T = T; p.D = D; p.I = I; p.ldo = ldo; p.ldw = ldw; p.lddx = ld_dx; p.w_out_in = out_in_of(dtype);
+  dtype = elem_of(dtype);
   hipStream_t s = (hipStream_t)stream;
   if (fsw::fast_path_ok_input_grad(p)) {
     const bool ws_ok = workspace && workspace_bytes > 0 && ((uintptr_t)workspace & 15) == 0;
@@ -195,20 +217,80 @@ int fsw_weight_grad(const void* x, const void* grad_xw_up, const void* grad_xw_g
     return fail(FSW_ERR_NULL_POINTER, "%s: all five arrays must be non-null", fn);
   if (!dtype_ok(dtype)) return fail(FSW_ERR_BAD_DTYPE, "%s: dtype %d is neither bf16 (0) nor fp16 (1)", fn, dtype);
   if (int e = check_dims(fn, T, D, I)) return e;
+  const bool oi = out_in_of(dtype);
+  dtype = elem_of(dtype);
   if (int e = check_ld(fn, "ldx", ldx, D)) return e;
   if (int e = check_ld(fn, "ldo", ldo, I)) return e;
-  if (int e = check_ld(fn, "ld_dw", ld_dw, I)) return e;
+  if (int e = check_ld(fn, "ld_dw", ld_dw, oi ? D : I)) return e;
   if (!al2(x) || !al2(grad_xw_up) || !al2(grad_xw_gate) || !al2(grad_w_up) || !al2(grad_w_gate))
     return fail(FSW_ERR_ALIGNMENT, "%s: pointers must be 2-byte aligned", fn);
   fsw::Problem p{};
   p.x = x; p.dG = grad_xw_gate; p.dU = grad_xw_up; p.dWg = grad_w_gate; p.dWu = grad_w_up;
-  p.T = T; p.D = D; p.I = I; p.ldx = ldx; p.ldo = ldo; p.lddw = ld_dw;
+  p.T = T; p.D = D; p.I = I; p.ldx = ldx; p.ldo = ldo; p.lddw = ld_dw; p.w_out_in = oi;
   hipStream_t s = (hipStream_t)stream;
   if (fsw::fast_path_ok_weight_grad(p)) {
     const bool ws_ok = workspace && workspace_bytes > 0 && ((uintptr_t)workspace & 15) == 0;
     return launched(fn, fsw::launch_weight_grad_fast(dtype, p, s, ws_ok ? workspace : nullptr, ws_ok ? workspace_bytes : 0));
   }
   return launched(fn, fsw::launch_weight_grad_generic(dtype, p, s));
+}
+
+// ---- the down projection that follows the SwiGLU: three plain GEMMs on the same tiled kernels ----
+static int run_gemm(const char* fn, int layout, const void* a, const void* b, void* c, int64_t M, int64_t N,
+                    int64_t K, int64_t lda, int64_t ldb, int64_t ldc, void* workspace, int64_t workspace_bytes,
+                    int dtype, void* stream) {
+  fsw::GemmProblem p{a, b, c, M, N, K, lda, ldb, ldc, layout};
+  hipStream_t s = (hipStream_t)stream;
+  if (fsw::fast_path_ok_gemm(p)) {
+    const bool ws_ok = workspace && workspace_bytes > 0 && ((uintptr_t)workspace & 15) == 0;
+    return launched(fn, fsw::launch_gemm_fast(dtype, p, s, ws_ok ? workspace : nullptr, ws_ok ? workspace_bytes : 0));
+  }
+  return launched(fn, fsw::launch_gemm_generic(dtype, p, s));
+}
+
+static int check_down_proj(const char* fn, const void* p0, const void* p1, const void* p2, int64_t T, int64_t I,
+                           int64_t D, int64_t ld_act, int64_t ldw, int64_t ldy, int dtype) {
+  if (!p0 || !p1 || !p2) return fail(FSW_ERR_NULL_POINTER, "%s: all three arrays must be non-null", fn);
+  if (!dtype_ok(dtype)) return fail(FSW_ERR_BAD_DTYPE, "%s: dtype %d is neither bf16 (0) nor fp16 (1)", fn, dtype);
+  if (int e = check_dims(fn, T, D, I)) return e;
+  if (int e = check_ld(fn, "ld_act", ld_act, I)) return e;
+  if (int e = check_ld(fn, "ldw", ldw, out_in_of(dtype) ? I : D)) return e;
+  if (int e = check_ld(fn, "ldy", ldy, D)) return e;
+  if (!al2(p0) || !al2(p1) || !al2(p2)) return fail(FSW_ERR_ALIGNMENT, "%s: pointers must be 2-byte aligned", fn);
+  return FSW_OK;
+}
+
+int fsw_down_proj_forward(const void* act, const void* w_down, void* y, int64_t T, int64_t I, int64_t D,
+                          int64_t ld_act, int64_t ldw, int64_t ldy, void* workspace, int64_t workspace_bytes,
+                          int dtype, void* stream) {
+  const char* fn = "fsw_down_proj_forward";
+  if (int e = check_down_proj(fn, act, w_down, y, T, I, D, ld_act, ldw, ldy, dtype)) return e;
+  // y [T,D] = act [T,I] W_down [I,D]   (or act W_down^T for W_down [D,I])
+  return run_gemm(fn, out_in_of(dtype) ? 1 : 0, act, w_down, y, T, D, I, ld_act, ldw, ldy, workspace, workspace_bytes,
+                  elem_of(dtype), stream);
+}
+
+int fsw_down_proj_input_grad(const void* grad_y, const void* w_down, void* grad_act, int64_t T, int64_t I,
+                             int64_t D, int64_t ldy, int64_t ldw, int64_t ld_act, void* workspace,
+                             int64_t workspace_bytes, int dtype, void* stream) {
+  const char* fn = "fsw_down_proj_input_grad";
+  if (int e = check_down_proj(fn, grad_y, w_down, grad_act, T, I, D, ld_act, ldw, ldy, dtype)) return e;
+  // grad_act [T,I] = grad_y [T,D] W_down^T   (or grad_y W_down for W_down [D,I])
+  return run_gemm(fn, out_in_of(dtype) ? 0 : 1, grad_y, w_down, grad_act, T, I, D, ldy, ldw, ld_act, workspace,
+                  workspace_bytes, elem_of(dtype), stream);
+}
+
+int fsw_down_proj_weight_grad(const void* act, const void* grad_y, void* grad_w_down, int64_t T, int64_t I,
+                              int64_t D, int64_t ld_act, int64_t ldy, int64_t ld_dw, void* workspace,
+                              int64_t workspace_bytes, int dtype, void* stream) {
+  const char* fn = "fsw_down_proj_weight_grad";
+  if (int e = check_down_proj(fn, act, grad_y, grad_w_down, T, I, D, ld_act, ld_dw, ldy, dtype)) return e;
+  // grad_W_down [I,D] = act^T grad_y   (or [D,I] = grad_y^T act)
+  if (out_in_of(dtype))
+    return run_gemm(fn, 2, grad_y, act, grad_w_down, D, I, T, ldy, ld_act, ld_dw, workspace, workspace_bytes,
+                    elem_of(dtype), stream);
+  return run_gemm(fn, 2, act, grad_y, grad_w_down, I, D, T, ld_act, ldy, ld_dw, workspace, workspace_bytes,
+                  elem_of(dtype), stream);
 }
 
 }  // extern "C"
@@ -254,7 +336,7 @@ int fsw_input_grad_noalloc(const void* grad_xw_gate, const void* grad_xw_up, con
   const char* fn = "fsw_input_grad_noalloc";
   if (int e = check_input_grad_args(fn, grad_xw_gate, grad_xw_up, w_gate, w_up, grad_x, T, D, I, ldo, ldw, ld_dx, dtype))
     return e;
-  const int64_t need = fsw::splitk_workspace_bytes(1, T, D, I);
+  const int64_t need = fsw::splitk_workspace_bytes(out_in_of(dtype) ? 4 : 1, T, D, I);
   if (need > (int64_t)FSW_NOALLOC_SCRATCH_BYTES)
     return fail(FSW_ERR_SCRATCH_LIMIT,
                 "%s: T=%lld D=%lld I=%lld needs %lld bytes of split-reduction scratch, the built-in buffer holds %lld; "

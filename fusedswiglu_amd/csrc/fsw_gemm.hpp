@@ -1,11 +1,20 @@
-// The tiled MFMA kernel behind the three GEMM-shaped steps of the SwiGLU path.
+// The tiled MFMA kernel behind every GEMM-shaped step of the SwiGLU path.  Weights are [D, I] ("in x out",
+// the reference's layout) in the first three modes and [I, D] (nn.Linear's layout) in the *T modes; the
+// three plain modes serve the down projection y = out W_down that follows the SwiGLU in an MLP.
 //
-//   kFwd  out = silu(x Wg) * (x Wu)      A = x [T,D] (k-contiguous), B = Wg | Wu [D,I] (n-contiguous)
-//   kDx   dx  = dG Wg^T + dU Wu^T        A = dG | dU [T,I] (k-contiguous), B = Wg | Wu [D,I] rows (k-contiguous)
-//   kDw   dWg = x^T dG, dWu = x^T dU     A = x [T,D] (m-contiguous), B = dG | dU [T,I] (n-contiguous)
+//   kFwd   out = silu(x Wg) * (x Wu)    A = x [T,D] (k-contiguous), B = Wg | Wu [D,I] (n-contiguous)
+//   kDx    dx  = dG Wg^T + dU Wu^T      A = dG | dU [T,I] (k-contiguous), B = Wg | Wu [D,I] rows (k-contiguous)
+//   kDw    dWg = x^T dG, dWu = x^T dU   A = x [T,D] (m-contiguous), B = dG | dU [T,I] (n-contiguous)
+//   kNN    C = A B                      A [M,K] k-contiguous, B [K,N] n-contiguous
+//   kNT    C = A B^T                    A [M,K] k-contiguous, B [N,K] k-contiguous
+//   kTN    C = A^T B                    A [K,M] m-contiguous, B [K,N] n-contiguous
+//   kFwdT  out = silu(x Wg^T) * (x Wu^T)   B = Wg | Wu [I,D] rows (k-contiguous)
+//   kDxT   dx  = dG Wg + dU Wu             B = Wg | Wu [I,D] (n-contiguous), two passes
+//   kDwT   dWg = dG^T x, dWu = dU^T x      A = dG | dU [T,I] (m-contiguous), B = x [T,D] (n-contiguous)
 //
-// One workgroup = 8 wavefronts (4 along M x 2 along N) = one 256 x 256 fp32 accumulator tile
-// (kFwd / kDw: 256 rows x 128 columns of EACH of the two results, sharing the A tile).
+// One workgroup = 8 wavefronts (4 along M x 2 along N) = one 256 x 256 fp32 accumulator tile (in the dual
+// modes 256 rows x 128 columns of EACH of the two results sharing the A tile; kDwT: 128 rows of each result
+// sharing the B tile).
 // The reduction advances 32 elements per step and is organised in PAIRS of steps.  Operand tiles are
 // brought in by direct global->LDS loads one to two pairs ahead of the MFMAs and kept in LDS rings
 // (A: three pairs, B: two pairs, 160 KiB in all):
@@ -21,39 +30,46 @@
 
 namespace fsw {
 
-enum Mode { kFwd = 0, kDx = 1, kDw = 2 };
+enum Mode { kFwd = 0, kDx = 1, kDw = 2, kNN = 3, kNT = 4, kTN = 5, kFwdT = 6, kDxT = 7, kDwT = 8 };
 
 struct GemmParams {
-  const void* a0;  // kFwd: x      kDx: dG     kDw: x
-  const void* a1;  //              kDx: dU
-  const void* b0;  // kFwd: Wg     kDx: Wg     kDw: dG
-  const void* b1;  // kFwd: Wu     kDx: Wu     kDw: dU
-  void* c0;        // kFwd: out    kDx: dx     kDw: dWg
-  void* c1;        // kFwd: g (may be null)    kDw: dWu
-  void* c2;        // kFwd: u (may be null)
-  // kFwd only, gating-gradient mode (d0 != null): nothing is written to c0; c1 = dG, c2 = dU with
+  const void* a0;  // kFwd*: x     kDx*: dG    kDw: x     kDwT: dG    plain: A
+  const void* a1;  //              kDx*: dU               kDwT: dU
+  const void* b0;  // kFwd*: Wg    kDx*: Wg    kDw: dG    kDwT: x     plain: B
+  const void* b1;  // kFwd*: Wu    kDx*: Wu    kDw: dU
+  void* c0;        // kFwd*: out   kDx*: dx    kDw*: dWg              plain: C
+  void* c1;        // kFwd*: g (may be null)   kDw*: dWu
+  void* c2;        // kFwd*: u (may be null)
+  // kFwd* only, gating-gradient mode (d0 != null): nothing is written to c0; c1 = dG, c2 = dU with
   // dU = d0 * silu(g), dG = d0 * u * silu'(g) computed from the fp32 accumulators (d0 has ldc too)
   const void* d0;
-  int M, N, K;     // GEMM view: kFwd (T,I,D)  kDx (T,D,I)  kDw (D,I,T)
+  int M, N, K;     // result rows x columns (per result) and reduction length (per pass)
   int lda, ldb, ldc;  // leading dimensions in elements
   int tiles_m, tiles_n, group_m;
-  // split-K (kDx, kDw on small problems): `splits` workgroups per tile each reduce `steps_per_split`
-  // steps (even) and store an fp32 partial tile to ws[split][M][N] (second result: + splits*M*N);
-  // fsw_splitk_reduce_kernel adds the partials in a fixed order.  splits == 1: results go to c0/c1.
+  // split-K (every mode but the forwards, on small problems): `splits` workgroups per tile each reduce
+  // `steps_per_split` steps (even) and store an fp32 partial tile to ws[split][M][N] (second result:
+  // + splits*M*N); fsw_splitk_reduce_kernel adds the partials in a fixed order.  splits == 1: results go
+  // to c0/c1.
   float* ws;
   int splits, steps_per_split;
 };
 
 constexpr int kThreads = 512;
-constexpr int kTileM = 256;
 constexpr int kMcSlotBytes = 2 * kMcPanelBytes;  // two 128-column panels: 16 KiB
 constexpr int kKcAreaBytes = 256 * 128;          // 256 rows x 64 k-elements: 32 KiB
 
 template <int MODE>
 struct Cfg {
-  static constexpr bool kAKc = (MODE != kDw);
-  static constexpr bool kBKc = (MODE == kDx);
-  static constexpr int kTileN = (MODE == kDx) ? 256 : 128;
+  static constexpr bool kAKc = !(MODE == kDw || MODE == kTN || MODE == kDwT);
+  static constexpr bool kBKc = (MODE == kDx || MODE == kNT || MODE == kFwdT);
+  static constexpr bool kForward = (MODE == kFwd || MODE == kFwdT);
+  static constexpr int kPasses = (MODE == kDx || MODE == kDxT) ? 2 : 1;
+  // two results that share the A tile (128 columns of each per tile) / the B tile (128 rows of each)
+  static constexpr bool kDualN = (MODE == kFwd || MODE == kDw || MODE == kFwdT);
+  static constexpr bool kDualM = (MODE == kDwT);
+  static constexpr int kResults = (MODE == kDw || MODE == kDwT) ? 2 : 1;
+  static constexpr int kTileM = kDualM ? 128 : 256;  // result rows / columns one tile covers
+  static constexpr int kTileN = kDualN ? 128 : 256;
   // rings in pairs of steps: 96 KiB for A, 64 KiB for B in either layout
   static constexpr int kPairsA = 3;
   static constexpr int kPairsB = 2;
@@ -92,14 +108,20 @@ FSW_DEV i16x8 read_frag_mc(const FSW_LDS char* panel, int block64, int ks, int l
 // MC panel of the tiled kernel: as above, and in k-rows with (k >> 3) odd the two 32-byte halves of
 // every 64-byte block are swapped.  16x16x32 operand (16 columns x 32 k-rows) by two transposing
 // reads: lane group g covers k-rows 8g .. 8g+7 (first read 8g..+3, second 8g+4..+7) of the same 16
-// columns, lane j of a group supplying columns (j & 3)*4.. of k-row (j >> 2).  Groups 0 and 1 (and 2
+// columns, lane j of a group supplying columns (j & 3)*8 bytes.. of k-row (j >> 2).  Groups 0 and 1 (and 2
 // and 3) then sit in different 32-byte halves, so each half-wave touches every bank once.
-FSW_DEV i16x8 read_frag_mc16(const FSW_LDS char* panel, int frag16, int lane) {
+// The byte address of fragment f (16-column block f of the panel) is
+//   krow*256 + (((f >> 1) ^ (j >> 2)) * 64) + (((f ^ grp) & 1) * 32) + (j & 3)*8  =  mc_lane_offset ^ (f << 5):
+// one per-lane offset serves every fragment, the fragment index only flips address bits 5..7.
+FSW_DEV unsigned mc_lane_offset(int lane) {
   const int grp = lane >> 4, j = lane & 15;
-  const int krow = 8 * grp + (j >> 2);
-  const int byte = krow * kMcRowBytes + (((frag16 >> 1) ^ (j >> 2)) * 64) + (((frag16 ^ grp) & 1) * 32) + (j & 3) * 8;
-  i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FSW_LDS i16x4*)(panel + byte));
-  i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FSW_LDS i16x4*)(panel + byte + 4 * kMcRowBytes));
+  return (unsigned)((8 * grp + (j >> 2)) * kMcRowBytes + (j >> 2) * 64 + (grp & 1) * 32 + (j & 3) * 8);
+}
+// `lane_ptr` = start of the panel (1 KiB aligned) + mc_lane_offset(lane)
+FSW_DEV i16x8 read_frag_mc16(const FSW_LDS char* lane_ptr, int frag16) {
+  const FSW_LDS char* q = (const FSW_LDS char*)(uintptr_t)((unsigned)(uintptr_t)lane_ptr ^ (unsigned)(frag16 << 5));
+  i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FSW_LDS i16x4*)q);
+  i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FSW_LDS i16x4*)(q + 4 * kMcRowBytes));
   i16x8 r;
   r.s0 = lo.x; r.s1 = lo.y; r.s2 = lo.z; r.s3 = lo.w;
   r.s4 = hi.x; r.s5 = hi.y; r.s6 = hi.z; r.s7 = hi.w;
@@ -107,19 +129,20 @@ FSW_DEV i16x8 read_frag_mc16(const FSW_LDS char* panel, int frag16, int lane) {
 }
 
 // ---- per-wave description of an operand's direct-to-LDS loads -----------------------
-// KC operand: a wave issues 4 instructions per area (rows 8*(wave + 8i) .. +8, 128 bytes each).
+// KC operand: a wave issues 4 instructions per area (tile rows 8*(wave + 8i) .. +8, 128 bytes each).
 struct KcLoader {
   unsigned lane_off;   // byte offset of this lane's 16 bytes for i = 0, relative to the moving base
-  unsigned row_step;   // bytes between the rows of consecutive i (64 rows)
+  unsigned row_step;   // bytes between the rows of consecutive i
   int klim[4];         // instruction i is in range while k0 < klim[i]
-  const char* base0;   // tile origin at k = 0 (first pass)
-  const char* base1;   // second pass (kDx), else the same
+  const char* base0;   // tile origin at k = 0: first pass / first matrix
+  const char* base1;   // second pass (kDx) or second matrix (kFwdT), else the same
 };
 // MC operand: 2 instructions per slot (wave, wave + 8): 4 k-rows x 256 bytes of panel (j >> 3).
 struct McLoader {
   unsigned lane_off[2];
   int klim[2];
-  const char* base[2];
+  const char* base[2];   // per panel
+  const char* base2[2];  // per panel, second pass (kDxT), else the same
   size_t kstep;  // bytes per 32 k-rows
 };
 
@@ -135,8 +158,24 @@ FSW_DEV void kc_setup(KcLoader& L, const void* p0, const void* p1, int row0, int
   L.base1 = (const char*)p1 + (size_t)row0 * ld * 2;
 }
 
-FSW_DEV void mc_setup(McLoader& L, const void* p_panel0, const void* p_panel1, int col0_panel0,
-                      int col0_panel1, int cols_total, int K, int ld, int wave, int lane) {
+// kFwdT: the 256 tile rows interleave the two weight matrices in blocks of 64 - instruction i fetches rows
+// row0 + 64*(i >> 1) + 8*wave.. of matrix (i & 1) - so that each wave's 128 B rows are 64 gate and 64 up
+// rows of the same output columns.
+FSW_DEV void kc_setup_interleaved(KcLoader& L, const void* p0, const void* p1, int row0, int rows_total,
+                                  int K, int ld, int wave, int lane) {
+  const int row = 8 * wave + (lane >> 3);
+  const int c = (lane & 7) ^ ((((wave & 1) << 2) + (lane >> 4)) & 7);
+  L.lane_off = (unsigned)row * (unsigned)ld * 2u + c * 16u;
+  L.row_step = 64u * (unsigned)ld * 2u;
+#pragma unroll
+  for (int i = 0; i < 4; i++) L.klim[i] = (row0 + row + 64 * (i >> 1) < rows_total) ? K - c * 8 : -0x40000000;
+  L.base0 = (const char*)p0 + (size_t)row0 * ld * 2;
+  L.base1 = (const char*)p1 + (size_t)row0 * ld * 2;
+}
+
+FSW_DEV void mc_setup(McLoader& L, const void* p_panel0, const void* p_panel1, const void* q_panel0,
+                      const void* q_panel1, int col0_panel0, int col0_panel1, int cols_total, int K, int ld,
+                      int wave, int lane) {
 #pragma unroll
   for (int i = 0; i < 2; i++) {
     const int j = wave + 8 * i;
@@ -147,6 +186,7 @@ FSW_DEV void mc_setup(McLoader& L, const void* p_panel0, const void* p_panel1, i
     L.lane_off[i] = (unsigned)row * (unsigned)ld * 2u + col * 2u;
     L.klim[i] = (col0 + col < cols_total) ? K - row : -0x40000000;
     L.base[i] = (const char*)((j >> 3) ? p_panel1 : p_panel0) + (size_t)col0 * 2;
+    L.base2[i] = (const char*)((j >> 3) ? q_panel1 : q_panel0) + (size_t)col0 * 2;
   }
   L.kstep = (size_t)kBK * ld * 2;
 }
@@ -156,7 +196,7 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
   using C = Cfg<MODE>;
   __shared__ __attribute__((aligned(1024))) char smem[C::kBytesA + C::kBytesB];
   constexpr bool A_KC = C::kAKc, B_KC = C::kBKc;
-  constexpr int TN = C::kTileN;
+  constexpr int TM = C::kTileM, TN = C::kTileN;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -164,17 +204,17 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
   const int wm = wave >> 1, wn = wave & 1;  // 4 waves along M x 2 along N
 
   const int ntiles = p.tiles_m * p.tiles_n;
-  const int split = (MODE == kFwd) ? 0 : (int)(blockIdx.x / ntiles);
+  const int split = C::kForward ? 0 : (int)(blockIdx.x / ntiles);
   const TileCoord tc = xcd_tile_order((int)(blockIdx.x - split * ntiles), p.tiles_m, p.tiles_n, p.group_m);
-  const int m0 = tc.tm * kTileM;
+  const int m0 = tc.tm * TM;
   const int n0 = tc.tn * TN;
 
-  // steps per pass; kDx makes two passes (dG.Wg^T then dU.Wu^T) and keeps pairs of steps inside a pass
-  const int kt1 = (MODE == kDx) ? (((p.K + kBK - 1) / kBK + 1) & ~1) : (p.K + kBK - 1) / kBK;
-  const int kt_all = (MODE == kDx) ? 2 * kt1 : kt1;
+  // steps per pass; the two-pass modes (dG.W then dU.W) keep pairs of steps inside a pass
+  const int kt1 = (C::kPasses == 2) ? (((p.K + kBK - 1) / kBK + 1) & ~1) : (p.K + kBK - 1) / kBK;
+  const int kt_all = C::kPasses * kt1;
   // this workgroup reduces steps kbase .. kbase + kt_total - 1 (everything unless split-K is on)
   const int kbase = split * p.steps_per_split;
-  const int kt_total = (MODE == kFwd) ? kt_all : min(p.steps_per_split, kt_all - kbase);
+  const int kt_total = C::kForward ? kt_all : min(p.steps_per_split, kt_all - kbase);
 
   const unsigned smem_a = (unsigned)(uintptr_t)(FSW_LDS char*)smem;
   const unsigned smem_b = smem_a + C::kBytesA;
@@ -183,62 +223,81 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
 
   KcLoader ka, kb;
   McLoader ma, mb;
-  if constexpr (A_KC) kc_setup(ka, p.a0, MODE == kDx ? p.a1 : p.a0, m0, p.M, p.K, p.lda, wave, lane);
-  else mc_setup(ma, p.a0, p.a0, m0, m0 + 128, p.M, p.K, p.lda, wave, lane);
-  if constexpr (B_KC) kc_setup(kb, p.b0, p.b1, n0, p.N, p.K, p.ldb, wave, lane);
-  else mc_setup(mb, p.b0, p.b1, n0, n0, p.N, p.K, p.ldb, wave, lane);
+  if constexpr (A_KC) kc_setup(ka, p.a0, C::kPasses == 2 ? p.a1 : p.a0, m0, p.M, p.K, p.lda, wave, lane);
+  else if constexpr (C::kDualM) mc_setup(ma, p.a0, p.a1, p.a0, p.a1, m0, m0, p.M, p.K, p.lda, wave, lane);
+  else mc_setup(ma, p.a0, p.a0, p.a0, p.a0, m0, m0 + 128, p.M, p.K, p.lda, wave, lane);
+  if constexpr (MODE == kFwdT) kc_setup_interleaved(kb, p.b0, p.b1, n0, p.N, p.K, p.ldb, wave, lane);
+  else if constexpr (B_KC) kc_setup(kb, p.b0, C::kPasses == 2 ? p.b1 : p.b0, n0, p.N, p.K, p.ldb, wave, lane);
+  else if constexpr (C::kDualN) mc_setup(mb, p.b0, p.b1, p.b0, p.b1, n0, n0, p.N, p.K, p.ldb, wave, lane);
+  else mc_setup(mb, p.b0, p.b0, C::kPasses == 2 ? p.b1 : p.b0, C::kPasses == 2 ? p.b1 : p.b0, n0, n0 + 128, p.N, p.K,
+                p.ldb, wave, lane);
 
   // Loads of the pair of steps (st, st+1), st even: four 1 KiB instructions per wave in either layout.
   // They are issued for EVERY pair index the loop asks for, also beyond the end of the reduction, where
   // every lane is out of range and zero-fills: the loop below is branch-free and its vmcnt arithmetic
   // never changes (and a last, odd step is multiplied by zeros).
-  auto kc_pair = [&](const KcLoader& L, int st, int pairs, unsigned lds_base) {
+  auto kc_pair = [&](const KcLoader& L, int st, int pairs, unsigned lds_base, bool interleaved) {
     const int apr = kbase + st;  // absolute step
-    const int pass = (MODE == kDx && apr >= kt1) ? 1 : 0;
+    const int pass = (C::kPasses == 2 && apr >= kt1) ? 1 : 0;
     const int k0 = (apr - pass * kt1) * kBK;
-    const i32x4 rs = make_rsrc((pass ? L.base1 : L.base0) + (size_t)k0 * 2);
     const unsigned dst = lds_base + (unsigned)((st >> 1) % pairs) * kKcAreaBytes + wave * 1024;
+    if (interleaved) {
+      const i32x4 rs0 = make_rsrc(L.base0 + (size_t)k0 * 2), rs1 = make_rsrc(L.base1 + (size_t)k0 * 2);
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const unsigned off = (k0 < L.klim[i]) ? L.lane_off + i * L.row_step : kOobOffset;
-      load16_to_lds(rs, off, dst + i * 8192);
+      for (int i = 0; i < 4; i++) {
+        const unsigned off = (k0 < L.klim[i]) ? L.lane_off + (i >> 1) * L.row_step : kOobOffset;
+        load16_to_lds((i & 1) ? rs1 : rs0, off, dst + i * 8192);
+      }
+    } else {
+      const i32x4 rs = make_rsrc((pass ? L.base1 : L.base0) + (size_t)k0 * 2);
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const unsigned off = (k0 < L.klim[i]) ? L.lane_off + i * L.row_step : kOobOffset;
+        load16_to_lds(rs, off, dst + i * 8192);
+      }
     }
   };
   auto mc_step = [&](const McLoader& L, int st, int pairs, unsigned lds_base) {
-    const int k0 = (kbase + st) * kBK;
+    const int apr = kbase + st;
+    const int pass = (C::kPasses == 2 && apr >= kt1) ? 1 : 0;
+    const int ks = apr - pass * kt1;  // step inside the pass
+    const int k0 = ks * kBK;
     const unsigned dst = lds_base + (unsigned)(st % (2 * pairs)) * kMcSlotBytes + wave * 1024;
 #pragma unroll
     for (int i = 0; i < 2; i++) {
       const unsigned off = (k0 < L.klim[i]) ? L.lane_off[i] : kOobOffset;
-      load16_to_lds(make_rsrc(L.base[i] + (size_t)(kbase + st) * L.kstep), off, dst + i * 8192);
+      load16_to_lds(make_rsrc((pass ? L.base2[i] : L.base[i]) + (size_t)ks * L.kstep), off, dst + i * 8192);
     }
   };
   auto issue_a = [&](int st) {
-    if constexpr (A_KC) kc_pair(ka, st, C::kPairsA, smem_a);
+    if constexpr (A_KC) kc_pair(ka, st, C::kPairsA, smem_a, false);
     else { mc_step(ma, st, C::kPairsA, smem_a); mc_step(ma, st + 1, C::kPairsA, smem_a); }
   };
   auto issue_b = [&](int st) {
-    if constexpr (B_KC) kc_pair(kb, st, C::kPairsB, smem_b);
+    if constexpr (B_KC) kc_pair(kb, st, C::kPairsB, smem_b, MODE == kFwdT);
     else { mc_step(mb, st, C::kPairsB, smem_b); mc_step(mb, st + 1, C::kPairsB, smem_b); }
   };
   // the 4 + 8 fragments of step kt (reading beyond the last step returns stale LDS bytes nobody uses)
+  const unsigned mc_off = mc_lane_offset(lane);
   auto read_frags = [&](int kt, i16x8 (&fq)[4], i16x8 (&fp)[8]) {
     const FSW_LDS char* ra;
     const FSW_LDS char* rb;
+    // MC: the per-lane offset is added to the (step-dependent) slot address here, so that the fragment
+    // addresses are recomputed with one XOR each instead of living in eight registers
     if constexpr (A_KC) ra = lds_a + ((kt >> 1) % C::kPairsA) * kKcAreaBytes;
-    else ra = lds_a + (kt % (2 * C::kPairsA)) * kMcSlotBytes;
+    else ra = lds_a + (kt % (2 * C::kPairsA)) * kMcSlotBytes + (wm >> 1) * kMcPanelBytes + mc_off;
     if constexpr (B_KC) rb = lds_b + ((kt >> 1) % C::kPairsB) * kKcAreaBytes;
-    else rb = lds_b + (kt % (2 * C::kPairsB)) * kMcSlotBytes;
+    else rb = lds_b + (kt % (2 * C::kPairsB)) * kMcSlotBytes + mc_off;
     const int half = kt & 1;
 #pragma unroll
     for (int mb = 0; mb < 4; mb++) {
       if constexpr (A_KC) fq[mb] = read_frag_kc16(ra, wm * 64 + mb * 16, half, lane);
-      else fq[mb] = read_frag_mc16(ra + (wm >> 1) * kMcPanelBytes, (wm & 1) * 4 + mb, lane);
+      else fq[mb] = read_frag_mc16(ra, (wm & 1) * 4 + mb);
     }
 #pragma unroll
     for (int nb = 0; nb < 8; nb++) {
       if constexpr (B_KC) fp[nb] = read_frag_kc16(rb, wn * 128 + nb * 16, half, lane);
-      else fp[nb] = read_frag_mc16(rb + (nb >> 2) * kMcPanelBytes, wn * 4 + (nb & 3), lane);
+      else fp[nb] = read_frag_mc16(rb + (nb >> 2) * kMcPanelBytes, wn * 4 + (nb & 3));
     }
   };
 
@@ -295,23 +354,38 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
   // the zero-filling loads beyond the end must have landed before the epilogue reuses LDS
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
-  // ---- epilogue.  acc[nb][mb][r] of lane l is row  wm*64 + mb*16 + (l & 15)  of the tile and column
-  // cbase(nb) + 4*(l >> 4) + r.  Each wave owns 64 consecutive columns (128 bytes) per result row, so
-  // it transposes 32 rows x 64 columns at a time through a private LDS patch and writes whole 128-byte
-  // lines: 8 rows x 128 bytes per store instruction.
-  if (MODE != kFwd && p.splits > 1) {
+  // ---- epilogue.  acc[nb][mb][r] of lane l is tile row  wm*64 + mb*16 + (l & 15)  and, within the wave's
+  // half h = nb >> 2, column (nb & 3)*16 + 4*(l >> 4) + r of 64 consecutive result columns (128 bytes).
+  // Where those 64 columns go (col_of_half) and which result a wave writes (result_of_half, row_base)
+  // depends on the mode.  Each wave transposes 32 rows x 64 columns at a time through a private LDS patch
+  // and writes whole 128-byte lines: 8 rows x 128 bytes per store instruction.
+  //   B k-contiguous (kDx, kNT): the wave's B rows wn*128 + h*64.. are result columns n0 + wn*128 + h*64..
+  //   dual-N (kFwd*, kDw): half h is result h (gate | up), columns n0 + wn*64..
+  //   one result from two B panels (kNN, kTN, kDxT, kDwT): columns n0 + h*128 + wn*64..
+  //   kDwT: waves with wm < 2 hold rows of the first result, the others of the second; 128 rows per tile
+  auto col_of_half = [&](int h) {
+    if constexpr (B_KC && MODE != kFwdT) return n0 + wn * 128 + h * 64;
+    else if constexpr (C::kDualN) return n0 + wn * 64;
+    else return n0 + h * 128 + wn * 64;
+  };
+  const int row_base = C::kDualM ? m0 + (wm & 1) * 64 : m0 + wm * 64;
+  auto result_of_half = [&](int h) -> int {
+    if constexpr (MODE == kDw) return h;
+    else if constexpr (C::kDualM) return wm >> 1;
+    else return 0;
+  };
+  if (!C::kForward && p.splits > 1) {
     // fp32 partial tile, 16 bytes (4 consecutive columns) per lane and store
     const size_t plane = (size_t)p.M * p.N;
 #pragma unroll
     for (int mb = 0; mb < 4; mb++) {
-      const int m = m0 + wm * 64 + mb * 16 + (lane & 15);
+      const int m = row_base + mb * 16 + (lane & 15);
       if (m >= p.M) continue;
 #pragma unroll
       for (int nb = 0; nb < 8; nb++) {
-        const int ncol = 4 * (lane >> 4);
-        const int n = (MODE == kDx) ? n0 + wn * 128 + nb * 16 + ncol : n0 + wn * 64 + (nb & 3) * 16 + ncol;
+        const int n = col_of_half(nb >> 2) + (nb & 3) * 16 + 4 * (lane >> 4);
         if (n >= p.N) continue;
-        const size_t which = (MODE == kDx) ? 0 : (size_t)(nb >> 2);
+        const size_t which = (size_t)result_of_half(nb >> 2);
         float* dst = p.ws + (which * p.splits + split) * plane + (size_t)m * p.N + n;
         *(f32x4*)dst = acc[nb][mb];
       }
@@ -327,7 +401,7 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const u32x4 v = *(const FSW_LDS u32x4*)(patch + rd_off + i * 8 * kPatchPitch);
-      const int m = m0 + wm * 64 + q * 32 + 8 * i + (lane >> 3);
+      const int m = row_base + q * 32 + 8 * i + (lane >> 3);
       const int n = col_base + (lane & 7) * 8;
       if (m < p.M && n < p.N) *(u32x4*)(dst + (size_t)m * p.ldc + n) = v;
     }
@@ -340,7 +414,7 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
   };
 #pragma unroll
   for (int q = 0; q < 2; q++) {  // 32 rows of the wave's 64 at a time
-    if constexpr (MODE == kFwd) {
+    if constexpr (C::kForward) {
       // gating-gradient mode: this lane's upstream gradients, 4 consecutive columns per 16x16 block
       u32x2 dv[2][4];
       const bool gating = p.d0 != nullptr;
@@ -349,7 +423,7 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
         for (int mbl = 0; mbl < 2; mbl++)
 #pragma unroll
           for (int c = 0; c < 4; c++) {
-            const int m = m0 + wm * 64 + (2 * q + mbl) * 16 + (lane & 15);
+            const int m = row_base + (2 * q + mbl) * 16 + (lane & 15);
             const int n = n0 + wn * 64 + c * 16 + 4 * (lane >> 4);
             dv[mbl][c] = (m < p.M && n < p.N) ? *(const u32x2*)((const unsigned short*)p.d0 + (size_t)m * p.ldc + n)
                                               : u32x2{0u, 0u};
@@ -384,9 +458,8 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
         flush_patch(dst, n0 + wn * 64, q);
       }
     } else {
-      constexpr int kHalves = 2;  // kDx: two 64-column halves of one result; kDw: gate and up results
 #pragma unroll
-      for (int h = 0; h < kHalves; h++) {
+      for (int h = 0; h < 2; h++) {  // the wave's two groups of 64 columns
 #pragma unroll
         for (int mbl = 0; mbl < 2; mbl++)
 #pragma unroll
@@ -394,8 +467,7 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
             const f32x4 t = acc[4 * h + c][2 * q + mbl];
             *(FSW_LDS u32x2*)(patch + wr_off + mbl * 16 * kPatchPitch + c * 32) = pack4(t[0], t[1], t[2], t[3]);
           }
-        if constexpr (MODE == kDx) flush_patch((unsigned short*)p.c0, n0 + wn * 128 + h * 64, q);
-        else flush_patch((unsigned short*)(h == 0 ? p.c0 : p.c1), n0 + wn * 64, q);
+        flush_patch((unsigned short*)(result_of_half(h) == 0 ? p.c0 : p.c1), col_of_half(h), q);
       }
     }
   }

@@ -114,7 +114,8 @@ hipError_t launch_forward_generic(int dtype, const Problem& p, hipStream_t s) {
   GenericParams g{};
   g.a[0] = (cus)p.x; g.b[0][0] = (cus)p.wg; g.b[0][1] = (cus)p.wu;
   g.c[0] = (us)p.out; g.c[1] = (us)p.g; g.c[2] = (us)p.u;
-  g.a_sm = p.ldx; g.a_sk = 1; g.b_sk = p.ldw; g.b_sn = 1; g.ldc = p.ldo;
+  g.a_sm = p.ldx; g.a_sk = 1; g.ldc = p.ldo;
+  if (p.w_out_in) { g.b_sk = 1; g.b_sn = p.ldw; } else { g.b_sk = p.ldw; g.b_sn = 1; }
   g.M = (int)p.T; g.N = (int)p.I; g.K = (int)p.D; g.passes = 1; g.dual = 1; g.swiglu = 1;
   if (p.dout) { g.swiglu = 2; g.dout = (cus)p.dout; }
   return launch_generic(dtype, g, s);
@@ -124,17 +125,36 @@ hipError_t launch_input_grad_generic(int dtype, const Problem& p, hipStream_t s)
   GenericParams g{};
   g.a[0] = (cus)p.dG; g.a[1] = (cus)p.dU; g.b[0][0] = (cus)p.wg; g.b[1][0] = (cus)p.wu;
   g.c[0] = (us)p.dx;
-  g.a_sm = p.ldo; g.a_sk = 1; g.b_sk = 1; g.b_sn = p.ldw; g.ldc = p.lddx;
+  g.a_sm = p.ldo; g.a_sk = 1; g.ldc = p.lddx;
+  if (p.w_out_in) { g.b_sk = p.ldw; g.b_sn = 1; } else { g.b_sk = 1; g.b_sn = p.ldw; }
   g.M = (int)p.T; g.N = (int)p.D; g.K = (int)p.I; g.passes = 2; g.dual = 0; g.swiglu = 0;
   return launch_generic(dtype, g, s);
 }
 
 hipError_t launch_weight_grad_generic(int dtype, const Problem& p, hipStream_t s) {
   GenericParams g{};
+  if (p.w_out_in) {  // results [I,D]: dW = dG^T x, one launch per result (this kernel shares A, not B)
+    g.b[0][0] = (cus)p.x; g.a_sm = 1; g.a_sk = p.ldo; g.b_sk = p.ldx; g.b_sn = 1; g.ldc = p.lddw;
+    g.M = (int)p.I; g.N = (int)p.D; g.K = (int)p.T; g.passes = 1; g.dual = 0; g.swiglu = 0;
+    g.a[0] = (cus)p.dG; g.c[0] = (us)p.dWg;
+    hipError_t e = launch_generic(dtype, g, s);
+    if (e != hipSuccess) return e;
+    g.a[0] = (cus)p.dU; g.c[0] = (us)p.dWu;
+    return launch_generic(dtype, g, s);
+  }
   g.a[0] = (cus)p.x; g.b[0][0] = (cus)p.dG; g.b[0][1] = (cus)p.dU;
   g.c[0] = (us)p.dWg; g.c[1] = (us)p.dWu;
   g.a_sm = 1; g.a_sk = p.ldx; g.b_sk = p.ldo; g.b_sn = 1; g.ldc = p.lddw;
   g.M = (int)p.D; g.N = (int)p.I; g.K = (int)p.T; g.passes = 1; g.dual = 1; g.swiglu = 0;
+  return launch_generic(dtype, g, s);
+}
+
+hipError_t launch_gemm_generic(int dtype, const GemmProblem& p, hipStream_t s) {
+  GenericParams g{};
+  g.a[0] = (cus)p.a; g.b[0][0] = (cus)p.b; g.c[0] = (us)p.c; g.ldc = p.ldc;
+  if (p.layout == 2) { g.a_sm = 1; g.a_sk = p.lda; } else { g.a_sm = p.lda; g.a_sk = 1; }
+  if (p.layout == 1) { g.b_sk = 1; g.b_sn = p.ldb; } else { g.b_sk = p.ldb; g.b_sn = 1; }
+  g.M = (int)p.M; g.N = (int)p.N; g.K = (int)p.K; g.passes = 1; g.dual = 0; g.swiglu = 0;
   return launch_generic(dtype, g, s);
 }
 

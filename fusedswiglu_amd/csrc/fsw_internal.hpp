@@ -19,7 +19,21 @@ struct Problem {
   long long T, D, I;
   long long ldx, ldw, ldo;       // leading dimensions (elements) of x, the weights, the [T,I] arrays
   long long lddx, lddw;          // of dx and of dWg/dWu
+  bool w_out_in;                 // weights and their gradients are [I,D] (nn.Linear's layout) instead of [D,I]
 };
+
+// A plain GEMM on the same kernels (the down projection that follows the SwiGLU and its two gradients).
+// layout 0: C = A B (A [M,K], B [K,N]); 1: C = A B^T (B [N,K]); 2: C = A^T B (A [K,M], B [K,N]); all row-major.
+struct GemmProblem {
+  const void *a, *b;
+  void* c;
+  long long M, N, K, lda, ldb, ldc;
+  int layout;
+};
+bool fast_path_ok_gemm(const GemmProblem& p);
+hipError_t launch_gemm_fast(int dtype, const GemmProblem& p, hipStream_t s, void* ws, long long ws_bytes);
+hipError_t launch_gemm_generic(int dtype, const GemmProblem& p, hipStream_t s);
+long long gemm_workspace_bytes(int layout, long long M, long long N, long long K);
 
 // Tiled direct-to-LDS MFMA kernels: need every dimension and leading dimension to be a multiple
 // of 8 elements and every pointer 16-byte aligned.
@@ -29,7 +43,8 @@ bool fast_path_ok_weight_grad(const Problem& p);
 hipError_t launch_forward_fast(int dtype, const Problem& p, hipStream_t s);
 hipError_t launch_input_grad_fast(int dtype, const Problem& p, hipStream_t s, void* ws, long long ws_bytes);
 hipError_t launch_weight_grad_fast(int dtype, const Problem& p, hipStream_t s, void* ws, long long ws_bytes);
-// Bytes of fp32 scratch that let small input-grad (step 1) / weight-grad (step 2) problems split their reduction.
+// Bytes of fp32 scratch that let small input-grad (step 1; 4 for [I,D] weights) / weight-grad (step 2; 5)
+// problems split their reduction.
 long long splitk_workspace_bytes(int step, long long T, long long D, long long I);
 
 // Weight-streaming forward for T <= 128 tokens (same eligibility as the tiled forward otherwise).

@@ -173,7 +173,7 @@ static hipError_t launch_skinny_t(const GemmParams& g, hipStream_t s) {
   return hipGetLastError();
 }
 
-bool skinny_forward_ok(const Problem& p) { return p.T <= kSkMaxRows && fast_path_ok_forward(p); }
+bool skinny_forward_ok(const Problem& p) { return !p.w_out_in && p.T <= kSkMaxRows && fast_path_ok_forward(p); }
 
 hipError_t launch_forward_skinny(int dtype, const Problem& p, hipStream_t s) {
   GemmParams g{};

@@ -15,6 +15,8 @@ static bool dims_ok(const Problem& p) {
          p.I < (1LL << 31);
 }
 
+// With [I,D] weights the roles of D and I as contiguous index swap for the weight operands, but both must be
+// multiples of 8 either way (x, dx are D-contiguous, the [T,I] arrays I-contiguous).
 bool fast_path_ok_forward(const Problem& p) {
   return dims_ok(p) && ld_ok(p.ldx) && ld_ok(p.ldw) && ld_out_ok(p.ldo) && al16(p.x) && al16(p.wg) &&
          al16(p.wu) && al16(p.out) && al16(p.g) && al16(p.u) && al16(p.dout);
@@ -69,27 +71,41 @@ static SplitPlan plan_split(long long tiles, int steps, long long M, long long N
 }
 static int steps_of(int mode, long long K) {
   int steps = (int)((K + kBK - 1) / kBK);
-  return mode == kDx ? 2 * ((steps + 1) & ~1) : steps;
+  return (mode == kDx || mode == kDxT) ? 2 * ((steps + 1) & ~1) : steps;
+}
+
+// Scratch for a GEMM of the given mode with results `results` x [M, N] and a reduction of K per pass.
+template <int MODE>
+static long long workspace_of(long long M, long long N, long long K) {
+  using C = Cfg<MODE>;
+  const long long tiles = ((M + C::kTileM - 1) / C::kTileM) * ((N + C::kTileN - 1) / C::kTileN);
+  const SplitPlan pl = plan_split_unbounded(tiles, steps_of(MODE, K), M, N, C::kResults);
+  return pl.splits > 1 ? (long long)pl.splits * M * N * 4 * C::kResults : 0;
 }
 
 long long splitk_workspace_bytes(int step, long long T, long long D, long long I) {
-  if (step == 1) {  // input_grad: result [T, D], reduction over 2*I
-    const long long tiles = ((T + kTileM - 1) / kTileM) * ((D + 255) / 256);
-    const SplitPlan pl = plan_split_unbounded(tiles, steps_of(kDx, I), T, D, 1);
-    return pl.splits > 1 ? (long long)pl.splits * T * D * 4 : 0;
+  switch (step) {
+    case 1: return workspace_of<kDx>(T, D, I);    // input_grad: result [T, D], reduction over 2*I
+    case 2: return workspace_of<kDw>(D, I, T);    // weight_grad: results 2 x [D, I], reduction over T
+    case 4: return workspace_of<kDxT>(T, D, I);   // the same two for [I, D] weights
+    case 5: return workspace_of<kDwT>(I, D, T);
+    default: return 0;
   }
-  if (step == 2) {  // weight_grad: results 2 x [D, I], reduction over T
-    const long long tiles = ((D + kTileM - 1) / kTileM) * ((I + 127) / 128);
-    const SplitPlan pl = plan_split_unbounded(tiles, steps_of(kDw, T), D, I, 2);
-    return pl.splits > 1 ? (long long)pl.splits * D * I * 4 * 2 : 0;
+}
+
+long long gemm_workspace_bytes(int layout, long long M, long long N, long long K) {
+  switch (layout) {
+    case 0: return workspace_of<kNN>(M, N, K);
+    case 1: return workspace_of<kNT>(M, N, K);
+    case 2: return workspace_of<kTN>(M, N, K);
+    default: return 0;
   }
-  return 0;
 }
 
 template <int MODE>
 static hipError_t launch(int dtype, GemmParams g, hipStream_t s, void* ws = nullptr, long long ws_bytes = 0) {
-  constexpr int TN = Cfg<MODE>::kTileN;
-  g.tiles_m = (g.M + kTileM - 1) / kTileM;
+  constexpr int TM = Cfg<MODE>::kTileM, TN = Cfg<MODE>::kTileN;
+  g.tiles_m = (g.M + TM - 1) / TM;
   g.tiles_n = (g.N + TN - 1) / TN;
   // Height of the bands of tile-rows an XCD walks (xcd_tile_order).  The A panels of the 8 bands in
   // flight (8 XCDs x group_m panels of 256 rows x K) should stay in the 256 MB memory-side cache while
@@ -97,8 +113,8 @@ static hipError_t launch(int dtype, GemmParams g, hipStream_t s, void* ws = null
   g.group_m = g.K > 4096 ? 4 : 8;
   const long long tiles = (long long)g.tiles_m * g.tiles_n;
   const int steps = steps_of(MODE, g.K);
-  const int results = (MODE == kDw) ? 2 : 1;
-  const SplitPlan pl = (MODE == kFwd) ? SplitPlan{1, steps}
+  const int results = Cfg<MODE>::kResults;
+  const SplitPlan pl = Cfg<MODE>::kForward ? SplitPlan{1, steps}
                                       : plan_split(tiles, steps, g.M, g.N, results, ws, ws_bytes);
   g.ws = (float*)ws; g.splits = pl.splits; g.steps_per_split = pl.steps_per_split;
   const long long grid = tiles * pl.splits;
@@ -123,7 +139,7 @@ hipError_t launch_forward_fast(int dtype, const Problem& p, hipStream_t s) {
   g.a0 = p.x; g.b0 = p.wg; g.b1 = p.wu; g.c0 = p.out; g.c1 = p.g; g.c2 = p.u; g.d0 = p.dout;
   g.M = (int)p.T; g.N = (int)p.I; g.K = (int)p.D;
   g.lda = (int)p.ldx; g.ldb = (int)p.ldw; g.ldc = (int)p.ldo;
-  return launch<kFwd>(dtype, g, s);
+  return p.w_out_in ? launch<kFwdT>(dtype, g, s) : launch<kFwd>(dtype, g, s);
 }
 
 hipError_t launch_input_grad_fast(int dtype, const Problem& p, hipStream_t s, void* ws, long long ws_bytes) {
@@ -131,15 +147,40 @@ hipError_t launch_input_grad_fast(int dtype, const Problem& p, hipStream_t s, vo
   g.a0 = p.dG; g.a1 = p.dU; g.b0 = p.wg; g.b1 = p.wu; g.c0 = p.dx;
   g.M = (int)p.T; g.N = (int)p.D; g.K = (int)p.I;
   g.lda = (int)p.ldo; g.ldb = (int)p.ldw; g.ldc = (int)p.lddx;
-  return launch<kDx>(dtype, g, s, ws, ws_bytes);
+  return p.w_out_in ? launch<kDxT>(dtype, g, s, ws, ws_bytes) : launch<kDx>(dtype, g, s, ws, ws_bytes);
 }
 
 hipError_t launch_weight_grad_fast(int dtype, const Problem& p, hipStream_t s, void* ws, long long ws_bytes) {
   GemmParams g{};
+  if (p.w_out_in) {  // dWg [I,D] = dG^T x: the two results share the B tile (x)
+    g.a0 = p.dG; g.a1 = p.dU; g.b0 = p.x; g.c0 = p.dWg; g.c1 = p.dWu;
+    g.M = (int)p.I; g.N = (int)p.D; g.K = (int)p.T;
+    g.lda = (int)p.ldo; g.ldb = (int)p.ldx; g.ldc = (int)p.lddw;
+    return launch<kDwT>(dtype, g, s, ws, ws_bytes);
+  }
   g.a0 = p.x; g.b0 = p.dG; g.b1 = p.dU; g.c0 = p.dWg; g.c1 = p.dWu;
   g.M = (int)p.D; g.N = (int)p.I; g.K = (int)p.T;
   g.lda = (int)p.ldx; g.ldb = (int)p.ldo; g.ldc = (int)p.lddw;
   return launch<kDw>(dtype, g, s, ws, ws_bytes);
+}
+
+bool fast_path_ok_gemm(const GemmProblem& p) {
+  return p.M > 0 && p.N > 0 && p.K > 0 && p.M < (1LL << 31) && p.N < (1LL << 31) && p.K < (1LL << 31) &&
+         // the contiguous index of each operand must be a multiple of 8 elements
+         mult8(p.layout == 2 ? p.M : p.K) && mult8(p.layout == 1 ? p.K : p.N) && mult8(p.N) &&
+         ld_ok(p.lda) && ld_ok(p.ldb) && ld_out_ok(p.ldc) && al16(p.a) && al16(p.b) && al16(p.c);
+}
+
+hipError_t launch_gemm_fast(int dtype, const GemmProblem& p, hipStream_t s, void* ws, long long ws_bytes) {
+  GemmParams g{};
+  g.a0 = p.a; g.b0 = p.b; g.c0 = p.c;
+  g.M = (int)p.M; g.N = (int)p.N; g.K = (int)p.K;
+  g.lda = (int)p.lda; g.ldb = (int)p.ldb; g.ldc = (int)p.ldc;
+  switch (p.layout) {
+    case 0: return launch<kNN>(dtype, g, s, ws, ws_bytes);
+    case 1: return launch<kNT>(dtype, g, s, ws, ws_bytes);
+    default: return launch<kTN>(dtype, g, s, ws, ws_bytes);
+  }
 }
 
 }  // namespace fsw

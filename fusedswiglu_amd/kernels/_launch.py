@@ -6,7 +6,11 @@ libfusedswiglu.  Mirrors the launcher seam of the reference
   * x may have any number (>= 1) of leading dimensions; they are flattened into T tokens
     (the reference insists on exactly 3-D input, kernels_bf16.py:178-180);
   * weight gradients come back already reduced over all tokens, shape [D, I];
-  * the input gradient has its own launcher instead of two torch matmuls (swiglu.py:45).
+  * the input gradient has its own launcher instead of two torch matmuls (swiglu.py:45);
+  * `weights_out_in=True` takes the weights (and returns their gradients) in nn.Linear's [I, D]
+    layout instead of the reference's [D, I] (README.md:26-27), without transposing anything;
+  * down_proj_forward / _input_grad / _weight_grad are the down projection that follows the SwiGLU
+    in an MLP block (the reference leaves it to the caller, README.md:25-38).
 """
 from __future__ import annotations
 
@@ -63,22 +67,31 @@ def _ld(t2: torch.Tensor) -> int:
     return t2.stride(0) if t2.shape[0] > 1 else t2.shape[1]
 
 
+def _code(dtype: torch.dtype, weights_out_in: bool) -> int:
+    return _DTYPE_CODE[dtype] | (_abi.WEIGHTS_OUT_IN if weights_out_in else 0)
+
+
+def _weight_dims(w: torch.Tensor, weights_out_in: bool) -> Tuple[int, int]:
+    """(D, I) of a gate/up weight in either layout."""
+    return (w.shape[1], w.shape[0]) if weights_out_in else (w.shape[0], w.shape[1])
+
+
 def fused_swiglu_fwd(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, dtype: torch.dtype,
-                     save_preactivations: bool = True
+                     save_preactivations: bool = True, weights_out_in: bool = False
                      ) -> Tuple[torch.Tensor, Optional[torch.Tensor], Optional[torch.Tensor]]:
     """out = silu(x @ w_gate) * (x @ w_up); returns (out, x@w_gate, x@w_up) like
     kernels_bf16.py:162-206.  With save_preactivations=False the two pre-activation arrays are
     neither allocated nor written and None is returned for them."""
     _require(x.ndim >= 2 and w_up.ndim == 2 and w_gate.ndim == 2,
              "Incorrect number of dimensions for LHS or RHS")
-    _require(x.shape[-1] == w_up.shape[0],
+    D, I = _weight_dims(w_up, weights_out_in)
+    _require(x.shape[-1] == D,
              f"Dimension mismatch. Expected x.shape[-1] ({x.shape[-1]}) to be equal to "
-             f"w_up.shape[0] ({w_up.shape[0]})")
+             f"w_up.shape[{1 if weights_out_in else 0}] ({D})")
     _require(w_up.shape == w_gate.shape, "Expected both weight matrices to have same shape")
     _require(x.dtype == dtype and w_gate.dtype == dtype and w_up.dtype == dtype,
              f"Expected {dtype} inputs and weights, got {x.dtype}, {w_gate.dtype}, {w_up.dtype}")
     dev = _check_device(x, w_gate, w_up)
-    D, I = w_up.shape
     _require(x.numel() > 0 and I > 0, "empty input")
     x2, wg, wu = _rows(x), _rows(w_gate), _rows(w_up)
     if _ld(wg) != _ld(wu):
@@ -92,7 +105,7 @@ def fused_swiglu_fwd(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, 
         _abi.check(_abi.lib().fsw_swiglu_forward(
             x2.data_ptr(), wg.data_ptr(), wu.data_ptr(), out.data_ptr(),
             g.data_ptr() if g is not None else None, u.data_ptr() if u is not None else None,
-            T, D, I, _ld(x2), _ld(wg), I, _DTYPE_CODE[dtype], _stream_ptr(dev)))
+            T, D, I, _ld(x2), _ld(wg), I, _code(dtype, weights_out_in), _stream_ptr(dev)))
     return out, g, u
 
 
@@ -117,17 +130,18 @@ def elementwise_backward(grad_output: torch.Tensor, xw_gate: torch.Tensor, xw_up
 
 
 def gating_grad_recompute(grad_output: torch.Tensor, x: torch.Tensor, w_gate: torch.Tensor,
-                          w_up: torch.Tensor, dtype: torch.dtype) -> Tuple[torch.Tensor, torch.Tensor]:
+                          w_up: torch.Tensor, dtype: torch.dtype,
+                          weights_out_in: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
     """(grad_xw_up, grad_xw_gate) like elementwise_backward, but from x and the weights: the
     pre-activations x@w_gate and x@w_up are recomputed in fp32 inside the kernel and never stored.
     For backward passes that did not save them (fused_swiglu/swiglu.py:28 saves them always)."""
     _require(x.ndim >= 2 and w_up.ndim == 2 and w_gate.ndim == 2,
              "Incorrect number of dimensions for LHS or RHS")
-    _require(x.shape[-1] == w_up.shape[0],
+    D, I = _weight_dims(w_up, weights_out_in)
+    _require(x.shape[-1] == D,
              f"Dimension mismatch. Expected x.shape[-1] ({x.shape[-1]}) to be equal to "
-             f"w_up.shape[0] ({w_up.shape[0]})")
+             f"w_up.shape[{1 if weights_out_in else 0}] ({D})")
     _require(w_up.shape == w_gate.shape, "Expected both weight matrices to have same shape")
-    D, I = w_up.shape
     _require(tuple(grad_output.shape) == tuple(x.shape[:-1]) + (I,),
              f"grad_output {tuple(grad_output.shape)} does not match x {tuple(x.shape)} and I = {I}")
     _require(all(t.dtype == dtype for t in (grad_output, x, w_gate, w_up)), f"Expected {dtype} tensors")
@@ -142,22 +156,22 @@ def gating_grad_recompute(grad_output: torch.Tensor, x: torch.Tensor, w_gate: to
     with torch.cuda.device(dev):
         _abi.check(_abi.lib().fsw_gating_grad_recompute(
             x2.data_ptr(), wg.data_ptr(), wu.data_ptr(), dout.data_ptr(), grad_xw_up.data_ptr(),
-            grad_xw_gate.data_ptr(), x2.shape[0], D, I, _ld(x2), _ld(wg), I, _DTYPE_CODE[dtype],
+            grad_xw_gate.data_ptr(), x2.shape[0], D, I, _ld(x2), _ld(wg), I, _code(dtype, weights_out_in),
             _stream_ptr(dev)))
     return grad_xw_up, grad_xw_gate
 
 
 def fused_input_grad(grad_xw_gate: torch.Tensor, grad_xw_up: torch.Tensor, w_gate: torch.Tensor,
-                     w_up: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+                     w_up: torch.Tensor, dtype: torch.dtype, weights_out_in: bool = False) -> torch.Tensor:
     """grad_x = grad_xw_gate @ w_gate.T + grad_xw_up @ w_up.T in one kernel (swiglu.py:45)."""
     _require(grad_xw_gate.shape == grad_xw_up.shape, "gate/up gradient shapes differ")
     _require(w_gate.ndim == 2 and w_gate.shape == w_up.shape,
              "Expected both weight matrices to have same shape")
-    _require(grad_xw_gate.shape[-1] == w_gate.shape[1], "Dimension mismatch between gradients and weights")
+    D, I = _weight_dims(w_gate, weights_out_in)
+    _require(grad_xw_gate.shape[-1] == I, "Dimension mismatch between gradients and weights")
     _require(all(t.dtype == dtype for t in (grad_xw_gate, grad_xw_up, w_gate, w_up)),
              f"Expected {dtype} tensors")
     dev = _check_device(grad_xw_gate, grad_xw_up, w_gate, w_up)
-    D, I = w_gate.shape
     dg, du, wg, wu = _rows(grad_xw_gate), _rows(grad_xw_up), _rows(w_gate), _rows(w_up)
     if _ld(dg) != _ld(du):
         dg, du = dg.contiguous(), du.contiguous()
@@ -166,18 +180,19 @@ def fused_input_grad(grad_xw_gate: torch.Tensor, grad_xw_up: torch.Tensor, w_gat
     T = dg.shape[0]
     grad_x = torch.empty(tuple(grad_xw_gate.shape[:-1]) + (D,), device=dev, dtype=dtype)
     with torch.cuda.device(dev):
-        ws, ws_bytes = _workspace(_abi.STEP_INPUT_GRAD, T, D, I, dev)
+        flag = _abi.WEIGHTS_OUT_IN if weights_out_in else 0
+        ws, ws_bytes = _workspace(_abi.STEP_INPUT_GRAD | flag, T, D, I, dev)
         _abi.check(_abi.lib().fsw_input_grad(
             dg.data_ptr(), du.data_ptr(), wg.data_ptr(), wu.data_ptr(), grad_x.data_ptr(),
             T, D, I, _ld(dg), _ld(wg), D, ws.data_ptr() if ws is not None else None, ws_bytes,
-            _DTYPE_CODE[dtype], _stream_ptr(dev)))
+            _code(dtype, weights_out_in), _stream_ptr(dev)))
     return grad_x
 
 
 def fused_weight_grad(x: torch.Tensor, grad_xw_up: torch.Tensor, grad_xw_gate: torch.Tensor,
                       dtype: torch.dtype,
-                      out: Optional[Tuple[torch.Tensor, torch.Tensor]] = None
-                      ) -> Tuple[torch.Tensor, torch.Tensor]:
+                      out: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+                      weights_out_in: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
     """(grad_w_up, grad_w_gate) = (x^T grad_xw_up, x^T grad_xw_gate), each [D, I], reduced over
     every token in fp32.  Same argument and return order as fused_bmm (kernels_bf16.py:385-412),
     with the batch sum of swiglu.py:56-57 folded in.  `out` = (grad_w_up, grad_w_gate) lets the
@@ -193,25 +208,91 @@ def fused_weight_grad(x: torch.Tensor, grad_xw_up: torch.Tensor, grad_xw_gate: t
         dg, du = dg.contiguous(), du.contiguous()
     T, D = x2.shape
     I = du.shape[1]
+    wshape = (I, D) if weights_out_in else (D, I)
     if out is None:
-        grad_w_up = torch.empty((D, I), device=dev, dtype=dtype)
-        grad_w_gate = torch.empty((D, I), device=dev, dtype=dtype)
+        grad_w_up = torch.empty(wshape, device=dev, dtype=dtype)
+        grad_w_gate = torch.empty(wshape, device=dev, dtype=dtype)
     else:
         grad_w_up, grad_w_gate = out
-        _require(tuple(grad_w_up.shape) == (D, I) and tuple(grad_w_gate.shape) == (D, I),
-                 f"weight-gradient outputs must be [{D}, {I}]")
+        _require(tuple(grad_w_up.shape) == wshape and tuple(grad_w_gate.shape) == wshape,
+                 f"weight-gradient outputs must be {list(wshape)}")
         _require(grad_w_up.dtype == dtype and grad_w_gate.dtype == dtype, f"Expected {dtype} tensors")
         _check_device(x, grad_w_up, grad_w_gate)
         _require(grad_w_up.stride(-1) == 1 and grad_w_gate.stride(-1) == 1 and _ld(grad_w_up) == _ld(grad_w_gate)
-                 and _ld(grad_w_up) >= I,
+                 and _ld(grad_w_up) >= wshape[1],
                  "weight-gradient outputs need unit inner stride and equal row strides")
     with torch.cuda.device(dev):
-        ws, ws_bytes = _workspace(_abi.STEP_WEIGHT_GRAD, T, D, I, dev)
+        flag = _abi.WEIGHTS_OUT_IN if weights_out_in else 0
+        ws, ws_bytes = _workspace(_abi.STEP_WEIGHT_GRAD | flag, T, D, I, dev)
         _abi.check(_abi.lib().fsw_weight_grad(
             x2.data_ptr(), du.data_ptr(), dg.data_ptr(), grad_w_up.data_ptr(), grad_w_gate.data_ptr(),
             T, D, I, _ld(x2), _ld(du), _ld(grad_w_up), ws.data_ptr() if ws is not None else None, ws_bytes,
-            _DTYPE_CODE[dtype], _stream_ptr(dev)))
+            _code(dtype, weights_out_in), _stream_ptr(dev)))
     return grad_w_up, grad_w_gate
+
+
+# ---- the down projection that follows the SwiGLU (w_down [I, D]; [D, I] with weights_out_in) ----
+def _down_dims(w_down: torch.Tensor, weights_out_in: bool) -> Tuple[int, int]:
+    _require(w_down.ndim == 2, "w_down must be 2-D")
+    return (w_down.shape[1], w_down.shape[0]) if weights_out_in else (w_down.shape[0], w_down.shape[1])  # (I, D)
+
+
+def down_proj_forward(act: torch.Tensor, w_down: torch.Tensor, dtype: torch.dtype,
+                      weights_out_in: bool = False) -> torch.Tensor:
+    """y = act @ w_down (act [..., I], w_down [I, D]; act @ w_down.T for w_down [D, I])."""
+    I, D = _down_dims(w_down, weights_out_in)
+    _require(act.ndim >= 2 and act.shape[-1] == I, f"Dimension mismatch: act {tuple(act.shape)} vs I = {I}")
+    _require(act.dtype == dtype and w_down.dtype == dtype, f"Expected {dtype} tensors")
+    dev = _check_device(act, w_down)
+    _require(act.numel() > 0 and D > 0, "empty input")
+    a2, w2 = _rows(act), _rows(w_down)
+    T = a2.shape[0]
+    y = torch.empty(tuple(act.shape[:-1]) + (D,), device=dev, dtype=dtype)
+    flag = _abi.WEIGHTS_OUT_IN if weights_out_in else 0
+    with torch.cuda.device(dev):
+        ws, ws_bytes = _workspace(_abi.STEP_DOWN_FORWARD | flag, T, D, I, dev)
+        _abi.check(_abi.lib().fsw_down_proj_forward(
+            a2.data_ptr(), w2.data_ptr(), y.data_ptr(), T, I, D, _ld(a2), _ld(w2), D,
+            ws.data_ptr() if ws is not None else None, ws_bytes, _code(dtype, weights_out_in), _stream_ptr(dev)))
+    return y
+
+
+def down_proj_input_grad(grad_y: torch.Tensor, w_down: torch.Tensor, dtype: torch.dtype,
+                         weights_out_in: bool = False) -> torch.Tensor:
+    """grad_act = grad_y @ w_down.T (grad_y [..., D])."""
+    I, D = _down_dims(w_down, weights_out_in)
+    _require(grad_y.ndim >= 2 and grad_y.shape[-1] == D, f"Dimension mismatch: grad_y {tuple(grad_y.shape)} vs D = {D}")
+    _require(grad_y.dtype == dtype and w_down.dtype == dtype, f"Expected {dtype} tensors")
+    dev = _check_device(grad_y, w_down)
+    g2, w2 = _rows(grad_y), _rows(w_down)
+    T = g2.shape[0]
+    grad_act = torch.empty(tuple(grad_y.shape[:-1]) + (I,), device=dev, dtype=dtype)
+    flag = _abi.WEIGHTS_OUT_IN if weights_out_in else 0
+    with torch.cuda.device(dev):
+        ws, ws_bytes = _workspace(_abi.STEP_DOWN_INPUT_GRAD | flag, T, D, I, dev)
+        _abi.check(_abi.lib().fsw_down_proj_input_grad(
+            g2.data_ptr(), w2.data_ptr(), grad_act.data_ptr(), T, I, D, _ld(g2), _ld(w2), I,
+            ws.data_ptr() if ws is not None else None, ws_bytes, _code(dtype, weights_out_in), _stream_ptr(dev)))
+    return grad_act
+
+
+def down_proj_weight_grad(act: torch.Tensor, grad_y: torch.Tensor, dtype: torch.dtype,
+                          weights_out_in: bool = False) -> torch.Tensor:
+    """grad_w_down = act^T grad_y over every token, [I, D] ([D, I] with weights_out_in), fp32 reduction."""
+    _require(act.shape[:-1] == grad_y.shape[:-1], f"Dimension mismatch: act {tuple(act.shape)} vs grad_y {tuple(grad_y.shape)}")
+    _require(act.dtype == dtype and grad_y.dtype == dtype, f"Expected {dtype} tensors")
+    dev = _check_device(act, grad_y)
+    a2, g2 = _rows(act), _rows(grad_y)
+    T, I = a2.shape
+    D = g2.shape[1]
+    grad_w = torch.empty((D, I) if weights_out_in else (I, D), device=dev, dtype=dtype)
+    flag = _abi.WEIGHTS_OUT_IN if weights_out_in else 0
+    with torch.cuda.device(dev):
+        ws, ws_bytes = _workspace(_abi.STEP_DOWN_WEIGHT_GRAD | flag, T, D, I, dev)
+        _abi.check(_abi.lib().fsw_down_proj_weight_grad(
+            a2.data_ptr(), g2.data_ptr(), grad_w.data_ptr(), T, I, D, _ld(a2), _ld(g2), grad_w.shape[1],
+            ws.data_ptr() if ws is not None else None, ws_bytes, _code(dtype, weights_out_in), _stream_ptr(dev)))
+    return grad_w
 
 
 def fused_bmm(x_t: torch.Tensor, grad_xw_up: torch.Tensor, grad_xw_gate: torch.Tensor,

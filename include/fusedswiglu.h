@@ -15,7 +15,7 @@
  *     arguments are leading dimensions (row pitches) in ELEMENTS.
  *   - Every pointer is a device pointer on the current HIP device.  The caller owns every
  *     buffer; the library never allocates, frees or keeps a pointer after returning.
- *   - `dtype` selects 16-bit storage: FSW_DTYPE_BF16 or FSW_DTYPE_FP16.  Products are
+ *   - `dtype` selects 16-bit storage: FSW_DTYPE_BF16 or FSW_DTYPE_FP16 (optionally | FSW_WEIGHTS_OUT_IN).  Products are
  *     accumulated in fp32 on the MFMA units for both (CDNA4 has no fp16-accumulate mode,
  *     so the reference's fp16 "fast accumulation" maps to fp32 accumulation).
  *   - `stream` is a hipStream_t (NULL = the default stream).  Calls only enqueue work; they
@@ -44,6 +44,13 @@ extern "C" {
 #define FSW_VERSION 200 /* major*10000 + minor*100 + patch */
 
 enum { FSW_DTYPE_BF16 = 0, FSW_DTYPE_FP16 = 1 };
+/* May be OR-ed into any `dtype` argument (and into the `step` of fsw_workspace_bytes): the weights of the
+ * call - w_gate, w_up, w_down and their gradients - are stored "out x in" like torch.nn.Linear.weight, i.e.
+ * w_gate, w_up [I, D] and w_down [D, I], instead of the reference's "in x out" ([D, I]; README.md:26-27,
+ * fused_swiglu/test_swiglu.py:30-35).  `ldw` / `ld_dw` are then leading dimensions of those arrays.  Nothing is
+ * transposed in memory: other tiled-kernel variants read and write the layout in place (the weight-streaming
+ * forward for T <= 128 exists for the default layout only). */
+#define FSW_WEIGHTS_OUT_IN 0x100
 
 enum {
   FSW_OK = 0,
@@ -108,7 +115,8 @@ FSW_API int fsw_gating_grad_recompute(const void* x, const void* w_gate, const v
  * chip (small d_model), several workgroups split the reduction of one tile, write fp32 partial
  * tiles to `workspace` (device memory owned by the caller, 16-byte aligned, contents irrelevant) and
  * a second kernel adds them in a fixed order.  fsw_workspace_bytes gives a sufficient size for
- * step 1 (input_grad) or 2 (weight_grad); with workspace == NULL or a smaller size the call still
+ * step 1 (input_grad), 2 (weight_grad), 4 / 5 / 6 (down projection forward / input grad / weight grad),
+ * each optionally | FSW_WEIGHTS_OUT_IN; with workspace == NULL or a smaller size the call still
  * works, just without the split.  Large problems never touch the workspace.
  */
 FSW_API int64_t fsw_workspace_bytes(int step, int64_t T, int64_t D, int64_t I);
@@ -150,6 +158,28 @@ FSW_API int fsw_weight_grad(const void* x, const void* grad_xw_up, const void* g
                     void* grad_w_up, void* grad_w_gate, int64_t T, int64_t D, int64_t I,
                     int64_t ldx, int64_t ldo, int64_t ld_dw, void* workspace, int64_t workspace_bytes,
                     int dtype, void* stream);
+
+/*
+ * The down projection that follows the SwiGLU in an MLP block, y = act W_down, and its two gradients, on the
+ * same tiled kernels.  The reference stops at FusedSwiGLU.apply (README.md:25-38: the caller multiplies by
+ * its own down weight); these three entry points are that next step for callers that want the whole block from
+ * one library.  act = the SwiGLU output.
+ *   act, grad_act [T,I] (ld_act)   w_down, grad_w_down [I,D] (ldw, ld_dw; [D,I] with FSW_WEIGHTS_OUT_IN)
+ *   y, grad_y [T,D] (ldy)
+ *   forward      y           = act W_down
+ *   input_grad   grad_act    = grad_y W_down^T
+ *   weight_grad  grad_w_down = act^T grad_y      (summed over all T tokens in fp32)
+ * `workspace` as for fsw_input_grad (steps 4, 5, 6 of fsw_workspace_bytes).
+ */
+FSW_API int fsw_down_proj_forward(const void* act, const void* w_down, void* y, int64_t T, int64_t I, int64_t D,
+                                  int64_t ld_act, int64_t ldw, int64_t ldy, void* workspace,
+                                  int64_t workspace_bytes, int dtype, void* stream);
+FSW_API int fsw_down_proj_input_grad(const void* grad_y, const void* w_down, void* grad_act, int64_t T, int64_t I,
+                                     int64_t D, int64_t ldy, int64_t ldw, int64_t ld_act, void* workspace,
+                                     int64_t workspace_bytes, int dtype, void* stream);
+FSW_API int fsw_down_proj_weight_grad(const void* act, const void* grad_y, void* grad_w_down, int64_t T, int64_t I,
+                                      int64_t D, int64_t ld_act, int64_t ldy, int64_t ld_dw, void* workspace,
+                                      int64_t workspace_bytes, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

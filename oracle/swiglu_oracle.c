@@ -115,3 +115,34 @@ void osw_backward(const double* x, const double* wg, const double* wu, const dou
   osw_input_grad(dG, dU, wg, wu, T, D, I, dx);
   osw_weight_grad(x, dG, dU, T, D, I, dWg, dWu);
 }
+
+/* The step after the path: the down projection y = act @ W_down that the reference leaves to its caller
+ * (README.md:25-38).  act [T,I], w [I,D] -> y [T,D]. */
+void osw_down_proj_forward(const double* act, const double* w, int64_t T, int64_t I, int64_t D, double* y) {
+#pragma omp parallel for schedule(static)
+  for (int64_t t = 0; t < T; t++)
+    for (int64_t d = 0; d < D; d++) {
+      double s = 0.0;
+      for (int64_t i = 0; i < I; i++) s += act[t * I + i] * w[i * D + d];
+      y[t * D + d] = s;
+    }
+}
+
+/* Its gradients: d_act = dy @ W^T [T,I], dW = act^T @ dy [I,D] summed over all tokens. */
+void osw_down_proj_backward(const double* act, const double* w, const double* dy, int64_t T, int64_t I,
+                            int64_t D, double* d_act, double* dw) {
+#pragma omp parallel for schedule(static)
+  for (int64_t t = 0; t < T; t++)
+    for (int64_t i = 0; i < I; i++) {
+      double s = 0.0;
+      for (int64_t d = 0; d < D; d++) s += dy[t * D + d] * w[i * D + d];
+      d_act[t * I + i] = s;
+    }
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < I; i++)
+    for (int64_t d = 0; d < D; d++) {
+      double s = 0.0;
+      for (int64_t t = 0; t < T; t++) s += act[t * I + i] * dy[t * D + d];
+      dw[i * D + d] = s;
+    }
+}

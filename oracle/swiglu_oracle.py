@@ -104,6 +104,36 @@ def swiglu_backward(x, w_gate, w_up, grad_output) -> Tuple[np.ndarray, np.ndarra
 
 
 # --------------------------------------------------------------------------
+# the step after the path: the down projection of the MLP block the reference's users build
+# --------------------------------------------------------------------------
+def down_proj_fwd(act, w_down) -> np.ndarray:
+    """y = act @ W_down, act [..., I], W_down [I, D].  The reference ends at the SwiGLU output and leaves this
+    multiplication to the caller (README.md:25-38: `output = FusedSwiGLU.apply(...)`); it is restated
+    here because the build offers it as the next step of the path."""
+    return np.asarray(act, dtype=np.float64) @ np.asarray(w_down, dtype=np.float64)
+
+
+def down_proj_backward(act, w_down, grad_y) -> Tuple[np.ndarray, np.ndarray]:
+    """(d_act, dW_down) of y = act @ W_down: d_act = dy @ W_down^T, dW_down = act^T @ dy summed over
+    every leading (token) dimension."""
+    act = np.asarray(act, dtype=np.float64)
+    w = np.asarray(w_down, dtype=np.float64)
+    dy = np.asarray(grad_y, dtype=np.float64)
+    I = act.shape[-1]
+    return dy @ w.T, act.reshape(-1, I).T @ dy.reshape(-1, dy.shape[-1])
+
+
+def mlp_fwd_bwd(x, w_gate, w_up, w_down, grad_y):
+    """The whole block y = (silu(x Wg) * (x Wu)) W_down and its gradients:
+    returns (y, dx, dWg, dWu, dW_down), composing swiglu_backward (swiglu.py:34-58) with the down projection."""
+    act = fused_swiglu_fwd(x, w_gate, w_up)[0]
+    y = down_proj_fwd(act, w_down)
+    d_act, dwd = down_proj_backward(act, w_down, grad_y)
+    dx, dwg, dwu = swiglu_backward(x, w_gate, w_up, d_act)
+    return y, dx, dwg, dwu, dwd
+
+
+# --------------------------------------------------------------------------
 # 16-bit rounding (numpy has no bf16) and the reference's rounding sequence
 # --------------------------------------------------------------------------
 def round_bf16(a) -> np.ndarray:
@@ -243,8 +273,10 @@ def c_lib():
         lib.osw_input_grad.argtypes = [dp, dp, dp, dp, i64, i64, i64, dp]
         lib.osw_weight_grad.argtypes = [dp, dp, dp, i64, i64, i64, dp, dp]
         lib.osw_backward.argtypes = [dp, dp, dp, dp, i64, i64, i64, dp, dp, dp, dp]
+        lib.osw_down_proj_forward.argtypes = [dp, dp, i64, i64, i64, dp]
+        lib.osw_down_proj_backward.argtypes = [dp, dp, dp, i64, i64, i64, dp, dp]
         for f in ("osw_forward", "osw_elementwise_backward", "osw_input_grad", "osw_weight_grad",
-                  "osw_backward"):
+                  "osw_backward", "osw_down_proj_forward", "osw_down_proj_backward"):
             getattr(lib, f).restype = None
         _C_LIB = lib
     return _C_LIB
@@ -286,3 +318,14 @@ def c_elementwise_backward(grad_output, xw_gate, xw_up):
     dU, dG = np.empty_like(dout), np.empty_like(dout)
     c_lib().osw_elementwise_backward(_p(dout), _p(g), _p(u), dout.size, _p(dU), _p(dG))
     return dU, dG
+
+
+def c_down_proj(act, w_down, grad_y):
+    """Naive-loop down projection; act [T,I], w_down [I,D], grad_y [T,D].  Returns (y, d_act, dW_down)."""
+    act, w, dy = _c64(act), _c64(w_down), _c64(grad_y)
+    T, I = act.shape
+    D = w.shape[1]
+    y, d_act, dw = np.empty((T, D)), np.empty((T, I)), np.empty((I, D))
+    c_lib().osw_down_proj_forward(_p(act), _p(w), T, I, D, _p(y))
+    c_lib().osw_down_proj_backward(_p(act), _p(w), _p(dy), T, I, D, _p(d_act), _p(dw))
+    return y, d_act, dw

@@ -104,6 +104,23 @@ def test_backward_validation(L):
     assert b"built-in buffer" in L.fsw_last_error()
     header = open(os.path.join(ROOT, "include", "fusedswiglu.h")).read()
     assert re.search(r"#define FSW_NOALLOC_SCRATCH_BYTES \(32u << 20\)", header) and _abi.NOALLOC_SCRATCH_BYTES == 32 << 20
+    # the weight-layout flag rides on dtype: it changes which dimension ldw / ld_dw must cover
+    OI = _abi.WEIGHTS_OUT_IN
+    f = L.fsw_swiglu_forward
+    assert f(P, P, P, P, P, P, 8, 8, 16, 8, 8, 16, 0 | OI, None) != 4    # [I,D] weights: ldw >= D = 8 is enough
+    assert f(P, P, P, P, P, P, 8, 16, 8, 16, 8, 8, 0 | OI, None) == 4    # ldw = 8 < D = 16
+    assert f(P, P, P, P, P, P, 8, 8, 8, 8, 8, 8, 0x200, None) == 2       # unknown flag
+    assert dx(P, P, P, P, P, 8, 16, 8, 8, 8, 16, None, 0, 1 | OI, None) == 4  # ldw < D
+    dn = L.fsw_down_proj_forward
+    assert dn(P, None, P, 8, 8, 8, 8, 8, 8, None, 0, 0, None) == 1
+    assert dn(P, P, P, 8, 16, 8, 16, 4, 8, None, 0, 0, None) == 4          # w_down [I,D]: ldw < D
+    assert dn(P, P, P, 8, 16, 8, 16, 8, 8, None, 0, OI, None) == 4         # w_down [D,I]: ldw < I
+    assert dn(P, P, P, 8, 16, 8, 8, 8, 8, None, 0, 0, None) == 4           # ld_act < I
+    assert L.fsw_down_proj_input_grad(P, P, P, 8, 8, 0, 8, 8, 8, None, 0, 0, None) == 3
+    assert L.fsw_down_proj_weight_grad(P, P, P, 8, 8, 8, 8, 8, 8, None, 0, 5, None) == 2
+    # few output tiles and long reductions ask for scratch in the down projection's gradients too
+    assert L.fsw_workspace_bytes(6, 8192, 256, 768) > 0 and L.fsw_workspace_bytes(6 | OI, 8192, 256, 768) > 0
+    assert L.fsw_workspace_bytes(4, 8192, 4096, 12288) == 0 and L.fsw_workspace_bytes(2 | OI, 8192, 4096, 12288) == 0
     dw = L.fsw_weight_grad
     assert dw(P, None, P, P, P, 8, 8, 8, 8, 8, 8, None, 0, 1, None) == 1
     assert dw(P, P, P, P, P, 8, 8, 8, 8, 8, 8, None, 0, -3, None) == 2
@@ -183,7 +200,7 @@ def test_package_exports():
 
     # the reference's two names first (fused_swiglu/__init__.py:1-2), then this build's additions
     assert fusedswiglu_amd.__all__[:2] == ["FusedSwiGLU", "FastAccumFusedSwiGLU"]
-    assert set(fusedswiglu_amd.__all__[2:]) == {"swiglu", "swiglu_packed", "SwiGLU"}
+    assert set(fusedswiglu_amd.__all__[2:]) == {"swiglu", "swiglu_packed", "down_proj", "swiglu_mlp", "SwiGLU", "SwiGLUMLP"}
     assert issubclass(FusedSwiGLU, torch.autograd.Function)
     assert issubclass(FastAccumFusedSwiGLU, torch.autograd.Function)
 

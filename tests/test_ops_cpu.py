@@ -21,6 +21,23 @@ def test_fake_implementations_give_shapes_and_dtypes():
             assert dx.shape == x.shape and dwg.shape == (16, 24) and dwu.numel() == 0
             dx, dw, rest = torch.ops.fusedswiglu_amd.swiglu_backward(out, x, w, w, out, out, False, True, True, True)
             assert dx.numel() == 0 and dw.shape == (16, 48) and rest.numel() == 0
+            # nn.Linear-style [I, D] weights
+            wt = torch.empty(24, 16, dtype=dtype, device="cuda")
+            out2, g2, _ = torch.ops.fusedswiglu_amd.swiglu_forward(x, wt, wt, True, True)
+            assert out2.shape == g2.shape == (2, 5, 24)
+            dx, dwg, dwu = torch.ops.fusedswiglu_amd.swiglu_backward(out, x, wt, wt, out, out, True, True, True, False, True)
+            assert dx.shape == x.shape and dwg.shape == dwu.shape == (24, 16)
+            dx, dw, rest = torch.ops.fusedswiglu_amd.swiglu_backward(out, x, wt, wt, out, out, True, True, True, True, True)
+            assert dw.shape == (48, 16) and rest.numel() == 0
+            # the down projection and its gradients, both layouts of w_down
+            for oi, wd_shape in ((False, (24, 16)), (True, (16, 24))):
+                wd = torch.empty(*wd_shape, dtype=dtype, device="cuda")
+                y = torch.ops.fusedswiglu_amd.down_proj_forward(out, wd, oi)
+                assert y.shape == (2, 5, 16) and y.dtype == dtype
+                da, dwd = torch.ops.fusedswiglu_amd.down_proj_backward(y, out, wd, True, True, oi)
+                assert da.shape == out.shape and dwd.shape == wd_shape
+                da, dwd = torch.ops.fusedswiglu_amd.down_proj_backward(y, out, wd, False, True, oi)
+                assert da.numel() == 0 and dwd.shape == wd_shape
 
 
 def test_module_parameters():
@@ -58,3 +75,26 @@ def test_module_from_and_to_linear():
         assert torch.equal(g2.weight, gate.weight) and torch.equal(u2.weight, up.weight)
     with pytest.raises(ValueError):
         fsw.SwiGLU.from_linear(torch.nn.Linear(8, 8), up)
+
+
+def test_module_keeps_the_linear_layout_without_copies():
+    gate = torch.nn.Linear(32, 48, bias=False, dtype=torch.bfloat16)
+    up = torch.nn.Linear(32, 48, bias=False, dtype=torch.bfloat16)
+    down = torch.nn.Linear(48, 32, bias=False, dtype=torch.bfloat16)
+    m = fsw.SwiGLU.from_linear(gate, up, keep_layout=True)
+    assert m.weights_out_in and m.w_gate is gate.weight and m.w_up is up.weight  # the same Parameters
+    assert (m.d_model, m.d_intermediate) == (32, 48)
+    g2, u2 = m.to_linear()
+    assert torch.equal(g2.weight, gate.weight) and torch.equal(u2.weight, up.weight)
+    p = fsw.SwiGLU.from_linear(gate, up, keep_layout=True, packed=True)
+    assert p.w_gate_up.shape == (96, 32) and torch.equal(p.w_gate_up[:48], gate.weight) and torch.equal(p.w_gate_up[48:], up.weight)
+    fresh = fsw.SwiGLU(32, 48, weights_out_in=True)
+    assert fresh.w_gate.shape == (48, 32)
+    mlp = fsw.SwiGLUMLP.from_linear(gate, up, down)
+    assert mlp.weights_out_in and mlp.w_down is down.weight and mlp.swiglu.w_gate is gate.weight
+    assert sorted(n for n, _ in mlp.named_parameters()) == ["swiglu.w_gate", "swiglu.w_up", "w_down"]
+    mlp2 = fsw.SwiGLUMLP.from_linear(gate, up, down, keep_layout=False)
+    assert mlp2.w_down.shape == (48, 32) and torch.equal(mlp2.w_down, down.weight.t())
+    assert fsw.SwiGLUMLP(32, 48).w_down.shape == (48, 32) and fsw.SwiGLUMLP(32, 48, weights_out_in=True).w_down.shape == (32, 48)
+    with pytest.raises(ValueError):
+        fsw.SwiGLUMLP.from_linear(gate, up, torch.nn.Linear(48, 32))

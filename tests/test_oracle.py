@@ -123,6 +123,48 @@ def test_backward_matches_finite_differences(oracle):
         assert np.allclose(num, grad, rtol=1e-6, atol=1e-8)
 
 
+# ---- the down projection and the whole MLP block --------------------------------------------------
+@pytest.mark.parametrize("T,D,I", RAGGED)
+def test_down_proj_c_loops_match_numpy(oracle, T, D, I):
+    rng = np.random.default_rng(T * 1000 + D)
+    act, w, dy = rng.standard_normal((T, I)), rng.standard_normal((I, D)) / I ** 0.5, rng.standard_normal((T, D))
+    y_c, da_c, dw_c = oracle.c_down_proj(act, w, dy)
+    da_n, dw_n = oracle.down_proj_backward(act, w, dy)
+    assert np.allclose(y_c, oracle.down_proj_fwd(act, w), rtol=1e-12, atol=1e-13)
+    assert np.allclose(da_c, da_n, rtol=1e-12, atol=1e-13) and np.allclose(dw_c, dw_n, rtol=1e-12, atol=1e-13)
+    assert dw_n.shape == (I, D) and da_n.shape == (T, I)
+
+
+def test_mlp_block_matches_autograd_fp64_and_finite_differences(oracle):
+    B, S, D, I = 2, 5, 12, 20
+    gen = lambda k: torch.Generator().manual_seed(k)
+    x = torch.randn(B, S, D, dtype=torch.float64, generator=gen(1), requires_grad=True)
+    wg = (torch.randn(D, I, dtype=torch.float64, generator=gen(2)) / D ** 0.5).requires_grad_()
+    wu = (torch.randn(D, I, dtype=torch.float64, generator=gen(3)) / D ** 0.5).requires_grad_()
+    wd = (torch.randn(I, D, dtype=torch.float64, generator=gen(4)) / I ** 0.5).requires_grad_()
+    dy = torch.randn(B, S, D, dtype=torch.float64, generator=gen(5))
+    y = torch.matmul(torch.nn.functional.silu(torch.matmul(x, wg)) * torch.matmul(x, wu), wd)
+    y.backward(dy)
+    n = lambda t: t.detach().numpy()
+    o_y, dx, dwg, dwu, dwd = oracle.mlp_fwd_bwd(n(x), n(wg), n(wu), n(wd), n(dy))
+    assert np.allclose(o_y, n(y), rtol=1e-12, atol=1e-13)
+    for got, want in ((dx, x.grad), (dwg, wg.grad), (dwu, wu.grad), (dwd, wd.grad)):
+        assert np.allclose(got, want.numpy(), rtol=1e-10, atol=1e-12)
+    # a transposed down weight or a dropped term must not pass: dW_down != (dy^T act)^T only by layout,
+    # and the gradient w.r.t. a single element agrees with a central difference
+    h, idx = 1e-6, (3, 7)
+    wp, wm = n(wd).copy(), n(wd).copy()
+    wp[idx] += h
+    wm[idx] -= h
+    loss = lambda w: float((oracle.down_proj_fwd(oracle.fused_swiglu_fwd(n(x), n(wg), n(wu))[0], w) * n(dy)).sum())
+    assert abs((loss(wp) - loss(wm)) / (2 * h) - dwd[idx]) < 1e-6 * max(1.0, abs(dwd[idx]))
+    # special case: an identity down weight (I == D) passes the SwiGLU output and gradient through
+    sq = np.random.default_rng(0).standard_normal((6, 8))
+    assert np.allclose(oracle.down_proj_fwd(sq, np.eye(8)), sq)
+    da, dw = oracle.down_proj_backward(sq, np.eye(8), sq)
+    assert np.allclose(da, sq) and np.allclose(dw, sq.T @ sq)
+
+
 # ---- invariants and special cases --------------------------------------------------------------
 def test_zero_gate_weights(oracle):
     T, D, I = 6, 8, 10

@@ -322,7 +322,10 @@ def test_extreme_aspect_ratios(oracle, shape):
     twg = (torch.randn(D, I, device=DEV, dtype=torch.float32, generator=g) / D ** 0.5).to(dtype)
     twu = (torch.randn(D, I, device=DEV, dtype=torch.float32, generator=g) / D ** 0.5).to(dtype)
     tdy = torch.randn(B, S, I, device=DEV, dtype=torch.float32, generator=g).to(dtype)
-    assert _abi.lib().fsw_uses_tiled_kernel(0, B * S, D, I, D, I, I, I, 16) == 1
+    # forward: the weight-streaming kernel up to 128 tokens (code 2), the tiled one beyond; gradients: tiled
+    assert _abi.lib().fsw_uses_tiled_kernel(0, B * S, D, I, D, I, I, I, 16) == (2 if B * S <= 128 else 1)
+    assert _abi.lib().fsw_uses_tiled_kernel(1, B * S, D, I, D, I, I, D, 16) == 1
+    assert _abi.lib().fsw_uses_tiled_kernel(2, B * S, D, I, D, I, I, I, 16) == 1
     out, dx, dwg, dwu = run_fwd_bwd(dtype, tx, twg, twu, tdy)
     for t in (out, dx, dwg, dwu):
         assert torch.isfinite(t).all()
