@@ -289,11 +289,6 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    # ---- the other configurations, the eager PyTorch step and the vendor GEMMs on the same box
-    if not args.no_extra:
-        del out, g, u, dG, dU, dx, dWg, dWu
-        result["other_configs"] = other_configs(dev, (x, wg, wu, dout))
-
     # ---- skinny-M forward (weight streaming, HBM bound), forward only, no pre-activation stores
     if not args.no_extra:
         D4, I4 = 8192, 28672
@@ -318,6 +313,11 @@ def main():
         result["skinny_forward"] = {"workload": "C4: bf16 forward, x [M,8192], Wg/Wu [8192,28672]", "bound": "hbm",
                                     "peak_gbs": PEAK_HBM_GBS, "runs": skinny}
         del w_sets
+
+    # ---- the other configurations, the eager PyTorch step and the vendor GEMMs on the same box
+    if not args.no_extra:
+        del out, g, u, dG, dU, dx, dWg, dWu
+        result["other_configs"] = other_configs(dev, (x, wg, wu, dout))
 
     # ---- CPU baseline: the eager fp32 SwiGLU of the reference's test on this machine's host cores
     if not args.no_cpu_baseline:

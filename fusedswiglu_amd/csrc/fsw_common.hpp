@@ -104,6 +104,19 @@ FSW_DEV void load16_to_lds(i32x4 rsrc, unsigned voffset, unsigned lds_addr) {
       : "memory");
 }
 
+// The same load with the non-temporal hint, for operands that are read exactly once per launch (the weights
+// of a forward with a single row of tiles): the lines are not kept in L2 or the memory-side cache, which
+// leaves those to the operand that is re-read and measurably raises the streaming rate from HBM.
+FSW_DEV void load16_to_lds_stream(i32x4 rsrc, unsigned voffset, unsigned lds_addr) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 3\n\t"
+      "buffer_load_dwordx4 %1, %2, 0 offen nt lds"
+      :
+      : "s"(lds_addr), "v"(voffset), "s"(rsrc)
+      : "memory");
+}
+
 template <int N>
 FSW_DEV void wait_vmcnt_and_barrier() {
   static_assert(N >= 0 && N < 64, "vmcnt is 6 bits");

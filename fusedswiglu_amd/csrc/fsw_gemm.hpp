@@ -26,6 +26,8 @@
 // in registers, so a pair's LDS space is released (and refilled) at the single barrier in the middle of
 // the pair, and the fragment reads of a step are always one step ahead of the MFMAs that consume them.
 #pragma once
+#include <type_traits>
+
 #include "fsw_common.hpp"
 
 namespace fsw {
@@ -191,7 +193,8 @@ FSW_DEV void mc_setup(McLoader& L, const void* p_panel0, const void* p_panel1, c
   L.kstep = (size_t)kBK * ld * 2;
 }
 
-template <typename E, int MODE>
+// STREAM_B: the B operand is read once by the whole launch (a single row of tiles): load it non-temporally
+template <typename E, int MODE, bool STREAM_B = false>
 __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
   using C = Cfg<MODE>;
   __shared__ __attribute__((aligned(1024))) char smem[C::kBytesA + C::kBytesB];
@@ -236,7 +239,8 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
   // They are issued for EVERY pair index the loop asks for, also beyond the end of the reduction, where
   // every lane is out of range and zero-fills: the loop below is branch-free and its vmcnt arithmetic
   // never changes (and a last, odd step is multiplied by zeros).
-  auto kc_pair = [&](const KcLoader& L, int st, int pairs, unsigned lds_base, bool interleaved) {
+  auto kc_pair = [&](const KcLoader& L, int st, int pairs, unsigned lds_base, bool interleaved, auto stream) {
+    constexpr bool kStream = decltype(stream)::value;
     const int apr = kbase + st;  // absolute step
     const int pass = (C::kPasses == 2 && apr >= kt1) ? 1 : 0;
     const int k0 = (apr - pass * kt1) * kBK;
@@ -246,18 +250,21 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
 #pragma unroll
       for (int i = 0; i < 4; i++) {
         const unsigned off = (k0 < L.klim[i]) ? L.lane_off + (i >> 1) * L.row_step : kOobOffset;
-        load16_to_lds((i & 1) ? rs1 : rs0, off, dst + i * 8192);
+        if constexpr (kStream) load16_to_lds_stream((i & 1) ? rs1 : rs0, off, dst + i * 8192);
+        else load16_to_lds((i & 1) ? rs1 : rs0, off, dst + i * 8192);
       }
     } else {
       const i32x4 rs = make_rsrc((pass ? L.base1 : L.base0) + (size_t)k0 * 2);
 #pragma unroll
       for (int i = 0; i < 4; i++) {
         const unsigned off = (k0 < L.klim[i]) ? L.lane_off + i * L.row_step : kOobOffset;
-        load16_to_lds(rs, off, dst + i * 8192);
+        if constexpr (kStream) load16_to_lds_stream(rs, off, dst + i * 8192);
+        else load16_to_lds(rs, off, dst + i * 8192);
       }
     }
   };
-  auto mc_step = [&](const McLoader& L, int st, int pairs, unsigned lds_base) {
+  auto mc_step = [&](const McLoader& L, int st, int pairs, unsigned lds_base, auto stream) {
+    constexpr bool kStream = decltype(stream)::value;
     const int apr = kbase + st;
     const int pass = (C::kPasses == 2 && apr >= kt1) ? 1 : 0;
     const int ks = apr - pass * kt1;  // step inside the pass
@@ -266,16 +273,20 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
 #pragma unroll
     for (int i = 0; i < 2; i++) {
       const unsigned off = (k0 < L.klim[i]) ? L.lane_off[i] : kOobOffset;
-      load16_to_lds(make_rsrc((pass ? L.base2[i] : L.base[i]) + (size_t)ks * L.kstep), off, dst + i * 8192);
+      const i32x4 rs = make_rsrc((pass ? L.base2[i] : L.base[i]) + (size_t)ks * L.kstep);
+      if constexpr (kStream) load16_to_lds_stream(rs, off, dst + i * 8192);
+      else load16_to_lds(rs, off, dst + i * 8192);
     }
   };
   auto issue_a = [&](int st) {
-    if constexpr (A_KC) kc_pair(ka, st, C::kPairsA, smem_a, false);
-    else { mc_step(ma, st, C::kPairsA, smem_a); mc_step(ma, st + 1, C::kPairsA, smem_a); }
+    constexpr std::false_type keep{};
+    if constexpr (A_KC) kc_pair(ka, st, C::kPairsA, smem_a, false, keep);
+    else { mc_step(ma, st, C::kPairsA, smem_a, keep); mc_step(ma, st + 1, C::kPairsA, smem_a, keep); }
   };
   auto issue_b = [&](int st) {
-    if constexpr (B_KC) kc_pair(kb, st, C::kPairsB, smem_b, MODE == kFwdT);
-    else { mc_step(mb, st, C::kPairsB, smem_b); mc_step(mb, st + 1, C::kPairsB, smem_b); }
+    constexpr std::bool_constant<STREAM_B> hint{};
+    if constexpr (B_KC) kc_pair(kb, st, C::kPairsB, smem_b, MODE == kFwdT, hint);
+    else { mc_step(mb, st, C::kPairsB, smem_b, hint); mc_step(mb, st + 1, C::kPairsB, smem_b, hint); }
   };
   // the 4 + 8 fragments of step kt (reading beyond the last step returns stale LDS bytes nobody uses)
   const unsigned mc_off = mc_lane_offset(lane);
@@ -403,7 +414,8 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
       const u32x4 v = *(const FSW_LDS u32x4*)(patch + rd_off + i * 8 * kPatchPitch);
       const int m = row_base + q * 32 + 8 * i + (lane >> 3);
       const int n = col_base + (lane & 7) * 8;
-      if (m < p.M && n < p.N) *(u32x4*)(dst + (size_t)m * p.ldc + n) = v;
+      // written once, read by a later kernel at the earliest: keep the lines out of the way of the operands
+      if (m < p.M && n < p.N) __builtin_nontemporal_store(v, (u32x4*)(dst + (size_t)m * p.ldc + n));
     }
   };
   auto pack4 = [&](float a, float b, float c, float d) {

@@ -5,7 +5,8 @@
 // keeps a ring of LDS stages (8 stages of 20 KiB for up to 64 rows, 6 of 24 KiB for 128)
 // filled by direct global->LDS loads.  x (a few MiB at most, L2 resident) rides along in the same
 // stages.  Each wave computes all BM rows x 32 columns of the gate and the up product and applies
-// silu(g)*u in registers.
+// silu(g)*u in registers.  Fragment reads of the next step overlap the MFMAs of the current one, and a
+// slot goes back to the loader as soon as its fragments are in registers.
 #include "fsw_gemm.hpp"
 #include "fsw_internal.hpp"
 
@@ -70,9 +71,9 @@ __global__ __launch_bounds__(kSkThreads) void fsw_skinny_forward_kernel(GemmPara
     w_base[i] = (const char*)((j >> 3) ? p.b1 : p.b0) + (size_t)n0 * 2;
   }
   const size_t w_kstep = (size_t)kBK * p.ldb * 2;
-  constexpr int kPerStage = C::kPerStage;
+  // Loads are issued for every slot index, also beyond the reduction (all lanes out of range -> zero fill, no
+  // memory traffic), so the number of loads in flight at each wait is one compile-time constant.
   auto issue = [&](int s) {
-    if (s >= kt_total) return;
     const int k0 = s * kBK;
     const unsigned st = smem_addr + (unsigned)(s % kSkStages) * kSkStage;
 #pragma unroll
@@ -84,7 +85,18 @@ __global__ __launch_bounds__(kSkThreads) void fsw_skinny_forward_kernel(GemmPara
     for (int i = 0; i < 4; i++) {
       const int j = wave + 4 * i;
       const unsigned off = (k0 < w_klim[i]) ? w_off[i] : kOobOffset;
-      load16_to_lds(make_rsrc(w_base[i] + (size_t)s * w_kstep), off, st + kSkABytes + j * 1024);
+      load16_to_lds_stream(make_rsrc(w_base[i] + (size_t)s * w_kstep), off, st + kSkABytes + j * 1024);
+    }
+  };
+  auto read_frags = [&](int s, i16x8 (&fq)[2][NQ], i16x8 (&fp)[2][2]) {
+    const FSW_LDS char* sa = smem_l + (s % kSkStages) * kSkStage;
+    const FSW_LDS char* sb = sa + kSkABytes;
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
+#pragma unroll
+      for (int q = 0; q < NQ; q++) fq[ks][q] = read_frag_x(sa, q * 32, ks, lane);
+#pragma unroll
+      for (int a = 0; a < 2; a++) fp[ks][a] = read_frag_mc(sb + a * kMcPanelBytes, wave, ks, lane);
     }
   };
 
@@ -95,40 +107,43 @@ __global__ __launch_bounds__(kSkThreads) void fsw_skinny_forward_kernel(GemmPara
     for (int q = 0; q < NQ; q++)
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[a][q][r] = 0.f;
-
+  auto mfmas = [&](const i16x8 (&fq)[2][NQ], const i16x8 (&fp)[2][2]) {
 #pragma unroll
-  for (int s = 0; s < kSkStages - 1; s++) issue(s);
-  for (int kt = 0; kt < kt_total; kt++) {
-    // stage kt landed?  up to kSkStages-2 younger stages may stay in flight
-    const int younger = min(kt_total - 1 - kt, kSkStages - 2);
-    switch (younger) {
-      case 6: wait_vmcnt_and_barrier<(kSkStages > 7 ? 6 : 0) * kPerStage>(); break;
-      case 5: wait_vmcnt_and_barrier<(kSkStages > 6 ? 5 : 0) * kPerStage>(); break;
-      case 4: wait_vmcnt_and_barrier<(kSkStages > 5 ? 4 : 0) * kPerStage>(); break;
-      case 3: wait_vmcnt_and_barrier<3 * kPerStage>(); break;
-      case 2: wait_vmcnt_and_barrier<2 * kPerStage>(); break;
-      case 1: wait_vmcnt_and_barrier<1 * kPerStage>(); break;
-      default: wait_vmcnt_and_barrier<0>(); break;
-    }
-    // The barrier also says every wave has finished reading stage kt-1, which the next loads overwrite: each
-    // of those fragment reads feeds an MFMA the wave issued before it reached the barrier, and an MFMA is
-    // not issued before its operands have returned from LDS.
-    issue(kt + kSkStages - 1);
-    const FSW_LDS char* sa = smem_l + (kt % kSkStages) * kSkStage;
-    const FSW_LDS char* sb = sa + kSkABytes;
-#pragma unroll
-    for (int ks = 0; ks < 2; ks++) {
-      i16x8 fq[NQ], fp[2];
-#pragma unroll
-      for (int q = 0; q < NQ; q++) fq[q] = read_frag_x(sa, q * 32, ks, lane);
-#pragma unroll
-      for (int a = 0; a < 2; a++) fp[a] = read_frag_mc(sb + a * kMcPanelBytes, wave, ks, lane);
+    for (int ks = 0; ks < 2; ks++)
 #pragma unroll
       for (int q = 0; q < NQ; q++)
 #pragma unroll
-        for (int a = 0; a < 2; a++) acc[a][q] = E::mfma(fp[a], fq[q], acc[a][q]);
-    }
+        for (int a = 0; a < 2; a++) acc[a][q] = E::mfma(fp[ks][a], fq[ks][q], acc[a][q]);
+  };
+
+  // Software pipeline over two register sets: the fragments of step kt+1 are read from LDS while the matrix
+  // cores work on step kt.  hand_over() waits until (a) this wave's loads of the next step have landed (all
+  // but the youngest kSkStages-2 stages) and (b) its own fragment reads of the current step have returned;
+  // the barrier extends both to the workgroup, so the current step's slot can be refilled at once, before
+  // the current step's products are even issued.  kSkStages-1 stages of weights stay in flight throughout.
+  constexpr int kInFlight = (kSkStages - 2) * C::kPerStage;
+  static_assert(kInFlight < 64, "vmcnt is 6 bits");
+  auto hand_over = [&]() {
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "n"(kInFlight) : "memory");
+  };
+#pragma unroll
+  for (int s = 0; s < kSkStages - 1; s++) issue(s);
+  i16x8 fq0[2][NQ], fp0[2][2], fq1[2][NQ], fp1[2][2];
+  wait_vmcnt_and_barrier<kInFlight>();  // step 0 has landed
+  read_frags(0, fq0, fp0);
+  issue(kSkStages - 1);
+  // an odd number of steps runs one more on zero-filled slots, which adds nothing
+  for (int kt = 0; kt < kt_total; kt += 2) {
+    hand_over();
+    issue(kt + kSkStages);
+    read_frags(kt + 1, fq1, fp1);
+    mfmas(fq0, fp0);
+    hand_over();
+    issue(kt + 1 + kSkStages);
+    read_frags(kt + 2, fq0, fp0);
+    mfmas(fq1, fp1);
   }
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // the zero-filling loads past the end
   // acc[a][q][r] of lane l: row q*32 + (l & 31), column n0 + wave*32 + 8*(r >> 2) + 4*(l >> 5) + (r & 3)
 #pragma unroll
   for (int q = 0; q < NQ; q++) {

@@ -119,7 +119,13 @@ static hipError_t launch(int dtype, GemmParams g, hipStream_t s, void* ws = null
   g.ws = (float*)ws; g.splits = pl.splits; g.steps_per_split = pl.steps_per_split;
   const long long grid = tiles * pl.splits;
   if (grid > 0x7fffffffLL) return hipErrorInvalidValue;
-  if (dtype == kDtypeBF16) fsw_gemm_kernel<BF16, MODE><<<(unsigned)grid, kThreads, 0, s>>>(g);
+  // a forward with a single row of tiles reads every weight byte exactly once: stream them past the caches
+  if (Cfg<MODE>::kForward && g.tiles_m == 1) {
+    if constexpr (Cfg<MODE>::kForward) {
+      if (dtype == kDtypeBF16) fsw_gemm_kernel<BF16, MODE, true><<<(unsigned)grid, kThreads, 0, s>>>(g);
+      else fsw_gemm_kernel<FP16, MODE, true><<<(unsigned)grid, kThreads, 0, s>>>(g);
+    }
+  } else if (dtype == kDtypeBF16) fsw_gemm_kernel<BF16, MODE><<<(unsigned)grid, kThreads, 0, s>>>(g);
   else fsw_gemm_kernel<FP16, MODE><<<(unsigned)grid, kThreads, 0, s>>>(g);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess || pl.splits == 1) return e;
