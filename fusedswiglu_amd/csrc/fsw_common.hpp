@@ -59,7 +59,9 @@ struct FP16 {
 };
 
 // silu(g) * u and the gating gradients, fp32 throughout, one rounding at the store.
-FSW_DEV float sigmoidf_fast(float z) { return __frcp_rn(1.0f + __expf(-z)); }
+// v_rcp_f32 (1 ulp) instead of a correctly rounded division: ten instructions fewer per value in epilogues
+// that are VALU bound, and far inside the rounding of the 16-bit results
+FSW_DEV float sigmoidf_fast(float z) { return __builtin_amdgcn_rcpf(1.0f + __expf(-z)); }
 FSW_DEV float silu_mul(float g, float u) { return g * sigmoidf_fast(g) * u; }
 // dU = dout * silu(g), dG = dout * u * silu'(g), silu'(z) = s + z*s*(1 - s), s = sigmoid(z)
 FSW_DEV void gating_grad(float dout, float g, float u, float& dU, float& dG) {

@@ -1,12 +1,13 @@
 // Weight-streaming forward for few tokens (T <= 128): out = silu(x Wg) * (x Wu).
 // With so few rows the step is bound by reading Wg and Wu once from HBM, not by the MFMAs, so this
 // kernel is built around keeping many weight bytes in flight per CU: one workgroup of 4 waves (one
-// per SIMD) owns 128 columns of both weight matrices, walks the whole reduction in steps of 32, and
-// keeps a ring of LDS stages (8 stages of 20 KiB for up to 64 rows, 6 of 24 KiB for 128)
-// filled by direct global->LDS loads.  x (a few MiB at most, L2 resident) rides along in the same
-// stages.  Each wave computes all BM rows x 32 columns of the gate and the up product and applies
-// silu(g)*u in registers.  Fragment reads of the next step overlap the MFMAs of the current one, and a
-// slot goes back to the loader as soon as its fragments are in registers.
+// per SIMD) owns 128 columns of both weight matrices, walks the whole reduction in stages of 64 and
+// keeps a ring of LDS stages filled by direct global->LDS loads (4 stages of 36 / 40 KiB up to 64 rows,
+// 3 of 48 KiB for 65-128 rows).  x (a few MiB at most, L2 resident) rides along in the same stages as
+// full 128-byte lines.  Each wave computes all BM rows x 32 columns of the gate and the up product and
+// applies silu(g)*u in registers.  The weight loads carry the non-temporal hint: bytes that are read once
+// then leave L2 and the memory-side cache to x.  Fragment reads of the next half stage overlap the MFMAs
+// of the current one, and a slot goes back to the loader as soon as its fragments are in registers.
 #include "fsw_gemm.hpp"
 #include "fsw_internal.hpp"
 
@@ -14,92 +15,108 @@ namespace fsw {
 
 constexpr int kSkThreads = 256;
 
-// Every stage holds an x tile of max(BM, 64) rows x 64 bytes (1 KiB loads of 16 rows, one or more
-// per wave; rows beyond T zero-filled) and a 16 KiB weight slot.
+// A stage holds 64 k-elements: BM rows of x, one full 128-byte line each, in the k-contiguous LDS format of the
+// tiled kernels (16-byte chunk c of row r at position c ^ ((r >> 1) & 7), read with ds_read_b128), and 32 KiB of
+// weights:
+//   weights [I, D] (W_KC; reduction index contiguous, the nn.Linear layout): 128 gate rows and 128 up rows of
+//     the workgroup's 128 output columns, one line each, same format as x;
+//   weights [D, I]: 64 k-rows x 256 bytes of both matrices in two of the tiled kernels' 16 KiB slots (two
+//     128-column panels of 32 k-rows each), read with the transposing ds_read_b64_tr_b16.
 template <int BM>
 struct SkCfg {
-  static constexpr int kRowsX = BM < 64 ? 64 : BM;
-  static constexpr int kXBytes = kRowsX * 64;
-  static constexpr int kXLoads = kRowsX / 64;            // per wave and stage
-  static constexpr int kStage = kXBytes + kMcSlotBytes;  // 20 / 24 KiB
-  static constexpr int kStages = (160 * 1024) / kStage;  // 8 / 6
-  static constexpr int kPerStage = kXLoads + 4;          // loads a wave issues per stage
+  static constexpr int kXBytes = BM * 128;
+  static constexpr int kXLoads = BM / 32;               // per wave and stage (8 rows x 128 bytes each)
+  static constexpr int kWBytes = 256 * 128;
+  static constexpr int kStage = kXBytes + kWBytes;
+  static constexpr int kStages = (160 * 1024) / kStage;
+  static constexpr int kPerStage = kXLoads + 8;
 };
 
-// x tile: BM rows x 64 bytes; chunk c of row r at position c ^ ((r >> 2) & 3) (see the MC/KC notes
-// in fsw_gemm.hpp; with 64-byte rows sixteen rows span the 64 banks when XOR-ed by (r >> 2)).
-FSW_DEV i16x8 read_frag_x(const FSW_LDS char* a, int row_base, int ks, int lane) {
+// rows row_base .. +31 (lane & 31), k = 16*ks + 8*(lane >> 5) .. +7 of the stage's 64
+FSW_DEV i16x8 read_frag_kc32(const FSW_LDS char* area, int row_base, int ks, int lane) {
   const int row = row_base + (lane & 31);
-  const int chunk = (ks * 2 + (lane >> 5)) ^ ((lane >> 2) & 3);
-  return *(const FSW_LDS i16x8*)(a + row * 64 + chunk * 16);
+  const int chunk = (ks * 2 + (lane >> 5)) ^ ((row >> 1) & 7);
+  return *(const FSW_LDS i16x8*)(area + row * 128 + chunk * 16);
 }
 
-template <typename E, int BM>
+template <typename E, int BM, bool W_KC>
 __global__ __launch_bounds__(kSkThreads) void fsw_skinny_forward_kernel(GemmParams p) {
   using C = SkCfg<BM>;
   constexpr int NQ = BM / 32;
-  constexpr int kSkStages = C::kStages, kSkStage = C::kStage, kSkABytes = C::kXBytes;
-  __shared__ __attribute__((aligned(1024))) char smem[kSkStages * kSkStage];
+  constexpr int kStages = C::kStages, kStage = C::kStage, kXBytes = C::kXBytes;
+  __shared__ __attribute__((aligned(1024))) char smem[kStages * kStage];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n0 = blockIdx.x * 128;
-  const int kt_total = (p.K + kBK - 1) / kBK;
+  const int st_total = (p.K + 63) / 64;
   const unsigned smem_addr = (unsigned)(uintptr_t)(FSW_LDS char*)smem;
   const FSW_LDS char* smem_l = (const FSW_LDS char*)smem;
 
-  // x: load j of wave w covers rows 64j + 16w .. +15 (4 lanes x 16 bytes per row)
-  unsigned xa_off[C::kXLoads];
-  int xa_klim[C::kXLoads];
+  // instruction idx covers area rows 8*idx .. +7; this wave issues idx = wave + 4*j
+  unsigned x_off[C::kXLoads];
+  int x_klim[C::kXLoads];
 #pragma unroll
   for (int j = 0; j < C::kXLoads; j++) {
-    const int row = 64 * j + 16 * wave + (lane >> 2);
-    const int c = (lane & 3) ^ ((lane >> 4) & 3);
-    xa_off[j] = (unsigned)row * (unsigned)p.lda * 2u + c * 16u;
-    xa_klim[j] = (row < p.M) ? p.K - c * 8 : -0x40000000;
+    const int row = 8 * (wave + 4 * j) + (lane >> 3);
+    const int c = (lane & 7) ^ ((row >> 1) & 7);
+    x_off[j] = (unsigned)row * (unsigned)p.lda * 2u + c * 16u;
+    x_klim[j] = (row < p.M) ? p.K - c * 8 : -0x40000000;
   }
-  // weights: 16 instructions per stage, 4 k-rows x 256 bytes each; instruction j -> panel j >> 3
-  unsigned w_off[4];
-  int w_klim[4];
-  const char* w_base[4];
+  unsigned w_off[8];
+  int w_klim[8];        // W_KC: in range while k0 < klim;  else: while k0 < klim as well (k-row bound)
+  const char* w_base[8];
 #pragma unroll
-  for (int i = 0; i < 4; i++) {
-    const int j = wave + 4 * i;
-    const int row = 4 * (j & 7) + (lane >> 4);
-    const int col = (((lane >> 2) & 3) ^ ((lane >> 4) & 3)) * 32 + (lane & 3) * 8;
-    w_off[i] = (unsigned)row * (unsigned)p.ldb * 2u + col * 2u;
-    w_klim[i] = (n0 + col < p.N) ? p.K - row : -0x40000000;
-    w_base[i] = (const char*)((j >> 3) ? p.b1 : p.b0) + (size_t)n0 * 2;
-  }
-  const size_t w_kstep = (size_t)kBK * p.ldb * 2;
-  // Loads are issued for every slot index, also beyond the reduction (all lanes out of range -> zero fill, no
-  // memory traffic), so the number of loads in flight at each wait is one compile-time constant.
-  auto issue = [&](int s) {
-    const int k0 = s * kBK;
-    const unsigned st = smem_addr + (unsigned)(s % kSkStages) * kSkStage;
-#pragma unroll
-    for (int j = 0; j < C::kXLoads; j++) {
-      const unsigned off = (k0 < xa_klim[j]) ? xa_off[j] : kOobOffset;
-      load16_to_lds(make_rsrc((const char*)p.a0 + (size_t)k0 * 2), off, st + j * 4096 + wave * 1024);
+  for (int j = 0; j < 8; j++) {
+    if constexpr (W_KC) {
+      const int row = 8 * (wave + 4 * j) + (lane >> 3);  // 0..255: gate rows, then up rows (j >= 4)
+      const int c = (lane & 7) ^ ((row >> 1) & 7);
+      const int n = row & 127;
+      w_off[j] = (unsigned)n * (unsigned)p.ldb * 2u + c * 16u;
+      w_klim[j] = (n0 + n < p.N) ? p.K - c * 8 : -0x40000000;
+      w_base[j] = (const char*)(j < 4 ? p.b0 : p.b1) + (size_t)n0 * p.ldb * 2;
+    } else {
+      // slot j >> 2 (k-rows 32*(j >> 2)..), instruction i = wave + 4*(j & 3) of its 16: panel i >> 3, 4 k-rows
+      const int i = wave + 4 * (j & 3);
+      const int row = 32 * (j >> 2) + 4 * (i & 7) + (lane >> 4);
+      const int col = (((lane >> 2) & 3) ^ ((lane >> 4) & 3)) * 32 + (lane & 3) * 8;
+      w_off[j] = (unsigned)row * (unsigned)p.ldb * 2u + col * 2u;
+      w_klim[j] = (n0 + col < p.N) ? p.K - row : -0x40000000;
+      w_base[j] = (const char*)((i >> 3) ? p.b1 : p.b0) + (size_t)n0 * 2;
     }
+  }
+  const size_t w_kstep = W_KC ? 128 : (size_t)64 * p.ldb * 2;  // bytes per stage along the reduction
+  // issued for every stage index; beyond the reduction every lane is out of range and zero-fills
+  auto issue = [&](int s) {
+    const int k0 = s * 64;
+    const unsigned st = smem_addr + (unsigned)(s % kStages) * kStage;
+    const i32x4 rx = make_rsrc((const char*)p.a0 + (size_t)k0 * 2);
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const int j = wave + 4 * i;
-      const unsigned off = (k0 < w_klim[i]) ? w_off[i] : kOobOffset;
-      load16_to_lds_stream(make_rsrc(w_base[i] + (size_t)s * w_kstep), off, st + kSkABytes + j * 1024);
+    for (int j = 0; j < C::kXLoads; j++)
+      load16_to_lds(rx, (k0 < x_klim[j]) ? x_off[j] : kOobOffset, st + (wave + 4 * j) * 1024);
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      // W_KC: area row block wave + 4*j;  else slot j >> 2, instruction wave + 4*(j & 3)
+      const unsigned dst = W_KC ? (unsigned)(wave + 4 * j) * 1024u
+                                : (unsigned)(j >> 2) * kMcSlotBytes + (unsigned)(wave + 4 * (j & 3)) * 1024u;
+      load16_to_lds_stream(make_rsrc(w_base[j] + (size_t)s * w_kstep), (k0 < w_klim[j]) ? w_off[j] : kOobOffset,
+                           st + kXBytes + dst);
     }
   };
-  auto read_frags = [&](int s, i16x8 (&fq)[2][NQ], i16x8 (&fp)[2][2]) {
-    const FSW_LDS char* sa = smem_l + (s % kSkStages) * kSkStage;
-    const FSW_LDS char* sb = sa + kSkABytes;
+  // half h of stage s: k = 32h .. 32h+31
+  auto read_frags = [&](int s, int h, i16x8 (&fq)[2][NQ], i16x8 (&fp)[2][2]) {
+    const FSW_LDS char* sx = smem_l + (s % kStages) * kStage;
+    const FSW_LDS char* sw = sx + kXBytes;
 #pragma unroll
     for (int ks = 0; ks < 2; ks++) {
 #pragma unroll
-      for (int q = 0; q < NQ; q++) fq[ks][q] = read_frag_x(sa, q * 32, ks, lane);
+      for (int q = 0; q < NQ; q++) fq[ks][q] = read_frag_kc32(sx, q * 32, 2 * h + ks, lane);
 #pragma unroll
-      for (int a = 0; a < 2; a++) fp[ks][a] = read_frag_mc(sb + a * kMcPanelBytes, wave, ks, lane);
+      for (int a = 0; a < 2; a++) {
+        if constexpr (W_KC) fp[ks][a] = read_frag_kc32(sw, a * 128 + wave * 32, 2 * h + ks, lane);
+        else fp[ks][a] = read_frag_mc(sw + h * kMcSlotBytes + a * kMcPanelBytes, wave, ks, lane);
+      }
     }
   };
-
   f32x16 acc[2][NQ];
 #pragma unroll
   for (int a = 0; a < 2; a++)
@@ -116,34 +133,27 @@ __global__ __launch_bounds__(kSkThreads) void fsw_skinny_forward_kernel(GemmPara
         for (int a = 0; a < 2; a++) acc[a][q] = E::mfma(fp[ks][a], fq[ks][q], acc[a][q]);
   };
 
-  // Software pipeline over two register sets: the fragments of step kt+1 are read from LDS while the matrix
-  // cores work on step kt.  hand_over() waits until (a) this wave's loads of the next step have landed (all
-  // but the youngest kSkStages-2 stages) and (b) its own fragment reads of the current step have returned;
-  // the barrier extends both to the workgroup, so the current step's slot can be refilled at once, before
-  // the current step's products are even issued.  kSkStages-1 stages of weights stay in flight throughout.
-  constexpr int kInFlight = (kSkStages - 2) * C::kPerStage;
+  // Per stage: read its second half while the first is multiplied; then one barrier, before which a wave
+  // waits for its loads of the next stage and for its own fragment reads of this one (both halves are in
+  // registers by then), so the slot can be refilled at once; read the next stage's first half while the
+  // second half is multiplied.
+  constexpr int kInFlight = (kStages - 2) * C::kPerStage;
   static_assert(kInFlight < 64, "vmcnt is 6 bits");
-  auto hand_over = [&]() {
-    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "n"(kInFlight) : "memory");
-  };
 #pragma unroll
-  for (int s = 0; s < kSkStages - 1; s++) issue(s);
+  for (int s = 0; s < kStages; s++) issue(s);
   i16x8 fq0[2][NQ], fp0[2][2], fq1[2][NQ], fp1[2][2];
-  wait_vmcnt_and_barrier<kInFlight>();  // step 0 has landed
-  read_frags(0, fq0, fp0);
-  issue(kSkStages - 1);
-  // an odd number of steps runs one more on zero-filled slots, which adds nothing
-  for (int kt = 0; kt < kt_total; kt += 2) {
-    hand_over();
-    issue(kt + kSkStages);
-    read_frags(kt + 1, fq1, fp1);
+  wait_vmcnt_and_barrier<(kStages - 1) * C::kPerStage>();  // stage 0 has landed
+  read_frags(0, 0, fq0, fp0);
+  for (int s = 0; s < st_total; s++) {
+    read_frags(s, 1, fq1, fp1);
     mfmas(fq0, fp0);
-    hand_over();
-    issue(kt + 1 + kSkStages);
-    read_frags(kt + 2, fq0, fp0);
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "n"(kInFlight) : "memory");
+    issue(s + kStages);
+    read_frags(s + 1, 0, fq0, fp0);
     mfmas(fq1, fp1);
   }
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // the zero-filling loads past the end
+
   // acc[a][q][r] of lane l: row q*32 + (l & 31), column n0 + wave*32 + 8*(r >> 2) + 4*(l >> 5) + (r & 3)
 #pragma unroll
   for (int q = 0; q < NQ; q++) {
@@ -175,27 +185,28 @@ __global__ __launch_bounds__(kSkThreads) void fsw_skinny_forward_kernel(GemmPara
   }
 }
 
-// Beyond 128 rows the 64-byte x rows of this kernel (as many bytes per step as the weights by then)
-// cost more than the deeper ring gains: the tiled kernel takes over (measured at 256 rows: 300 vs 258 us).
+// Beyond 128 rows a stage (x as many bytes as the weights by then) leaves room for two slots only: the tiled
+// kernel takes over.
 constexpr int kSkMaxRows = 128;
 
-template <typename E>
+template <typename E, bool W_KC>
 static hipError_t launch_skinny_t(const GemmParams& g, hipStream_t s) {
   const unsigned tiles = (unsigned)((g.N + 127) / 128);
-  if (g.M <= 32) fsw_skinny_forward_kernel<E, 32><<<tiles, kSkThreads, 0, s>>>(g);
-  else if (g.M <= 64) fsw_skinny_forward_kernel<E, 64><<<tiles, kSkThreads, 0, s>>>(g);
-  else fsw_skinny_forward_kernel<E, 128><<<tiles, kSkThreads, 0, s>>>(g);
+  if (g.M <= 32) fsw_skinny_forward_kernel<E, 32, W_KC><<<tiles, kSkThreads, 0, s>>>(g);
+  else if (g.M <= 64) fsw_skinny_forward_kernel<E, 64, W_KC><<<tiles, kSkThreads, 0, s>>>(g);
+  else fsw_skinny_forward_kernel<E, 128, W_KC><<<tiles, kSkThreads, 0, s>>>(g);
   return hipGetLastError();
 }
 
-bool skinny_forward_ok(const Problem& p) { return !p.w_out_in && p.T <= kSkMaxRows && fast_path_ok_forward(p); }
+bool skinny_forward_ok(const Problem& p) { return p.T <= kSkMaxRows && fast_path_ok_forward(p); }
 
 hipError_t launch_forward_skinny(int dtype, const Problem& p, hipStream_t s) {
   GemmParams g{};
   g.a0 = p.x; g.b0 = p.wg; g.b1 = p.wu; g.c0 = p.out; g.c1 = p.g; g.c2 = p.u;
   g.M = (int)p.T; g.N = (int)p.I; g.K = (int)p.D;
   g.lda = (int)p.ldx; g.ldb = (int)p.ldw; g.ldc = (int)p.ldo;
-  return dtype == kDtypeBF16 ? launch_skinny_t<BF16>(g, s) : launch_skinny_t<FP16>(g, s);
+  if (p.w_out_in) return dtype == kDtypeBF16 ? launch_skinny_t<BF16, true>(g, s) : launch_skinny_t<FP16, true>(g, s);
+  return dtype == kDtypeBF16 ? launch_skinny_t<BF16, false>(g, s) : launch_skinny_t<FP16, false>(g, s);
 }
 
 }  // namespace fsw

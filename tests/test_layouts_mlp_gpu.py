@@ -155,6 +155,33 @@ def test_mlp_module_from_linear(oracle, dtype, keep_layout):
     assert oracle.rel_error(np64(y), np64(ref)) < 2 * tol
 
 
+FEW_TOKENS = [(1, 8, 8), (7, 72, 136), (16, 520, 392), (33, 1032, 136), (64, 200, 1160), (65, 64, 264), (128, 1096, 520)]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("out_in", [False, True], ids=["DI", "ID"])
+@pytest.mark.parametrize("tdi", FEW_TOKENS, ids=lambda s: "x".join(map(str, s)))
+def test_few_token_forward_in_both_layouts(oracle, dtype, out_in, tdi):
+    """Up to 128 tokens the forward runs on the weight-streaming kernels (selection code 2), one per weight
+    layout: out and the saved pre-activations against the oracle, with reductions that are not multiples of a
+    stage (64 or 32 elements), ragged last column blocks and row counts on both sides of every variant."""
+    T, D, I = tdi
+    x, wg, wu, _, _, _ = make(oracle, (1, T, D, I), dtype, seed=T + D)
+    tx = dev(x[0], dtype)
+    twg, twu = (dev(wg.T, dtype), dev(wu.T, dtype)) if out_in else (dev(wg, dtype), dev(wu, dtype))
+    ldw = D if out_in else I
+    flag = _abi.WEIGHTS_OUT_IN if out_in else 0
+    assert _abi.lib().fsw_uses_tiled_kernel(flag, T, D, I, D, ldw, I, I, 16) == 2
+    out, g, u = _launch.fused_swiglu_fwd(tx, twg, twu, dtype, weights_out_in=out_in)
+    out_only = _launch.fused_swiglu_fwd(tx, twg, twu, dtype, save_preactivations=False, weights_out_in=out_in)[0]
+    torch.cuda.synchronize()
+    o_out, o_g, o_u = oracle.fused_swiglu_fwd(x[0], wg, wu)
+    tol = TOL[dtype]
+    assert oracle.rel_error(np64(out), o_out) < tol
+    assert oracle.rel_error(np64(g), o_g) < tol and oracle.rel_error(np64(u), o_u) < tol
+    assert torch.equal(out, out_only)
+
+
 def test_linear_layout_full_size_forward_slices(oracle):
     """The headline shape with nn.Linear-layout weights: whole token rows of out against the oracle."""
     dtype, T, D, I = torch.bfloat16, 8192, 4096, 12288
