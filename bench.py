@@ -294,24 +294,33 @@ def main():
         D4, I4 = 8192, 28672
         w_sets = [((torch.randn(D4, I4, device=dev, dtype=dt) / D4 ** 0.5), (torch.randn(D4, I4, device=dev, dtype=dt) / D4 ** 0.5))
                   for _ in range(2)]
-        skinny = []
-        for M in (16, 64, 128, 256):
-            xs = torch.randn(M, D4, device=dev, dtype=dt)
-            os_ = torch.empty(M, I4, device=dev, dtype=dt)
-            state = {"i": 0}
 
-            def fwd():
-                a, b = w_sets[state["i"] & 1]  # alternate weight sets: nothing stays cache resident
-                state["i"] += 1
-                _abi.check(L.fsw_swiglu_forward(p(xs), p(a), p(b), p(os_), None, None, M, D4, I4, D4, I4, I4, 0, stream))
+        def stream_runs(sets, flag, ldw):
+            runs = []
+            for M in (16, 64, 128, 256):
+                xs = torch.randn(M, D4, device=dev, dtype=dt)
+                os_ = torch.empty(M, I4, device=dev, dtype=dt)
+                state = {"i": 0}
 
-            ms = gpu_time_ms(fwd, iters=20)
-            nbytes = 2.0 * (2 * D4 * I4 + M * D4 + M * I4)
-            skinny.append({"M": M, "ms": round(ms, 4), "gbs": round(nbytes / ms / 1e6, 1),
-                           "frac_hbm_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4),
-                           "tflops": round(4.0 * M * D4 * I4 / ms / 1e9, 1)})
+                def fwd():
+                    a, b = sets[state["i"] & 1]  # alternate weight sets: nothing stays cache resident
+                    state["i"] += 1
+                    _abi.check(L.fsw_swiglu_forward(p(xs), p(a), p(b), p(os_), None, None, M, D4, I4, D4, ldw, I4, flag, stream))
+
+                ms = gpu_time_ms(fwd, iters=20)
+                nbytes = 2.0 * (2 * D4 * I4 + M * D4 + M * I4)
+                runs.append({"M": M, "ms": round(ms, 4), "gbs": round(nbytes / ms / 1e6, 1),
+                             "frac_hbm_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4),
+                             "tflops": round(4.0 * M * D4 * I4 / ms / 1e9, 1)})
+            return runs
+
+        skinny = stream_runs(w_sets, 0, I4)
+        # the same weights viewed as [I, D] storage (the values do not matter for the timing)
+        skinny_out_in = stream_runs([(a.view(I4, D4), b.view(I4, D4)) for a, b in w_sets], _abi.WEIGHTS_OUT_IN, D4)
         result["skinny_forward"] = {"workload": "C4: bf16 forward, x [M,8192], Wg/Wu [8192,28672]", "bound": "hbm",
-                                    "peak_gbs": PEAK_HBM_GBS, "runs": skinny}
+                                    "peak_gbs": PEAK_HBM_GBS, "runs": skinny,
+                                    "workload_weights_out_in": "the same with Wg/Wu stored [28672,8192] (nn.Linear layout)",
+                                    "runs_weights_out_in": skinny_out_in}
         del w_sets
 
     # ---- the other configurations, the eager PyTorch step and the vendor GEMMs on the same box
