@@ -403,15 +403,26 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
     }
     return;
   }
-  constexpr int kPatchPitch = 144;  // 128 + 16: keeps 16-byte alignment, spreads rows over banks
+  // patch: 32 rows x 128 bytes per wave; 16-byte chunk c of row r sits at position c ^ ((r >> 1) & 7), which
+  // keeps both the 8-byte accumulator writes (16 rows x 4 column groups per instruction) and the 16-byte
+  // row reads (2 rows x 128 bytes per 16 lanes) free of bank conflicts
+  constexpr int kPatchPitch = 128;
   FSW_LDS char* patch = (FSW_LDS char*)smem + wave * (32 * kPatchPitch);
-  const int wr_off = (lane & 15) * kPatchPitch + (lane >> 4) * 8;       // + mbl*16*pitch + c*32
-  const int rd_off = (lane >> 3) * kPatchPitch + (lane & 7) * 16;       // + i*8*pitch
+  const int wr_row = (lane & 15) * kPatchPitch, wr_swz = (lane >> 1) & 7, wr_grp = lane >> 4;
+  // 8 bytes of column group wr_grp of 16-column block c:  chunk 2c + (wr_grp >> 1), half wr_grp & 1
+  auto wr_off = [&](int mbl, int c) {
+    return mbl * 16 * kPatchPitch + wr_row + (((2 * c + (wr_grp >> 1)) ^ wr_swz) << 4) + (wr_grp & 1) * 8;
+  };
+  // row 8i + (lane >> 3), chunk lane & 7
+  auto rd_off = [&](int i) {
+    const int row = 8 * i + (lane >> 3);
+    return row * kPatchPitch + (((lane & 7) ^ ((row >> 1) & 7)) << 4);
+  };
   auto flush_patch = [&](unsigned short* dst, int col_base, int q) {
     // rows q*32 + 8i + (lane >> 3), columns col_base + (lane & 7)*8 .. +8
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-      const u32x4 v = *(const FSW_LDS u32x4*)(patch + rd_off + i * 8 * kPatchPitch);
+      const u32x4 v = *(const FSW_LDS u32x4*)(patch + rd_off(i));
       const int m = row_base + q * 32 + 8 * i + (lane >> 3);
       const int n = col_base + (lane & 7) * 8;
       // written once, read by a later kernel at the earliest: keep the lines out of the way of the operands
@@ -464,7 +475,7 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
                 v[e] = which == 0 ? silu_mul(g[e], u[e]) : (which == 1 ? g[e] : u[e]);
               }
             }
-            *(FSW_LDS u32x2*)(patch + wr_off + mbl * 16 * kPatchPitch + c * 32) = pack4(v[0], v[1], v[2], v[3]);
+            *(FSW_LDS u32x2*)(patch + wr_off(mbl, c)) = pack4(v[0], v[1], v[2], v[3]);
           }
         unsigned short* dst = (unsigned short*)(which == 0 ? p.c0 : (which == 1 ? p.c1 : p.c2));
         flush_patch(dst, n0 + wn * 64, q);
@@ -477,7 +488,7 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
 #pragma unroll
           for (int c = 0; c < 4; c++) {
             const f32x4 t = acc[4 * h + c][2 * q + mbl];
-            *(FSW_LDS u32x2*)(patch + wr_off + mbl * 16 * kPatchPitch + c * 32) = pack4(t[0], t[1], t[2], t[3]);
+            *(FSW_LDS u32x2*)(patch + wr_off(mbl, c)) = pack4(t[0], t[1], t[2], t[3]);
           }
         flush_patch((unsigned short*)(result_of_half(h) == 0 ? p.c0 : p.c1), col_of_half(h), q);
       }
