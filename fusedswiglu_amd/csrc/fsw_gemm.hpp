@@ -496,12 +496,16 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
   }
 }
 
-// out[i] = round(sum over s of ws[s][i]), i < n, fixed order: deterministic.  n is a multiple of 4.
+// out_r[i] = round(sum over s of ws[r][s][i]), i < n, fixed order: deterministic.  n is a multiple of 4.
+// blockIdx.y = result r (the weight gradients come in pairs): one launch for both.
 template <typename E>
-__global__ __launch_bounds__(256) void fsw_splitk_reduce_kernel(const float* __restrict__ ws, unsigned short* __restrict__ out,
-                                                                size_t n, int splits, int N, int ldc) {
+__global__ __launch_bounds__(256) void fsw_splitk_reduce_kernel(const float* __restrict__ ws, unsigned short* __restrict__ out0,
+                                                                unsigned short* __restrict__ out1, size_t n, int splits,
+                                                                int N, int ldc) {
   const size_t i4 = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
   if (i4 >= n) return;
+  ws += (size_t)blockIdx.y * splits * n;
+  unsigned short* out = blockIdx.y ? out1 : out0;
   f32x4 a = *(const f32x4*)(ws + i4);
   for (int s = 1; s < splits; s++) {
     const f32x4 b = *(const f32x4*)(ws + (size_t)s * n + i4);

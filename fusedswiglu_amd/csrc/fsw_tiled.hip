@@ -130,13 +130,13 @@ static hipError_t launch(int dtype, GemmParams g, hipStream_t s, void* ws = null
   hipError_t e = hipGetLastError();
   if (e != hipSuccess || pl.splits == 1) return e;
   const size_t n = (size_t)g.M * g.N;
-  const unsigned blocks = (unsigned)((n / 4 + 255) / 256);
-  for (int r = 0; r < results; r++) {
-    const float* src = (const float*)ws + (size_t)r * pl.splits * n;
-    unsigned short* dst = (unsigned short*)(r == 0 ? g.c0 : g.c1);
-    if (dtype == kDtypeBF16) fsw_splitk_reduce_kernel<BF16><<<blocks, 256, 0, s>>>(src, dst, n, pl.splits, g.N, g.ldc);
-    else fsw_splitk_reduce_kernel<FP16><<<blocks, 256, 0, s>>>(src, dst, n, pl.splits, g.N, g.ldc);
-  }
+  const dim3 blocks((unsigned)((n / 4 + 255) / 256), (unsigned)results);
+  if (dtype == kDtypeBF16)
+    fsw_splitk_reduce_kernel<BF16><<<blocks, 256, 0, s>>>((const float*)ws, (unsigned short*)g.c0, (unsigned short*)g.c1, n,
+                                                         pl.splits, g.N, g.ldc);
+  else
+    fsw_splitk_reduce_kernel<FP16><<<blocks, 256, 0, s>>>((const float*)ws, (unsigned short*)g.c0, (unsigned short*)g.c1, n,
+                                                         pl.splits, g.N, g.ldc);
   return hipGetLastError();
 }
 

@@ -42,8 +42,33 @@ def _check_device(*tensors: torch.Tensor) -> torch.device:
     return dev
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream_ptr(dev: torch.device) -> int:
+    """Handle of torch's current HIP stream on `dev` (without building a Stream object when torch offers
+    the raw getter: this runs four times per training step)."""
+    if _raw_stream is not None and dev.index is not None:
+        return _raw_stream(dev.index)
     return torch.cuda.current_stream(dev).cuda_stream
+
+
+class _on_device:
+    """`with torch.cuda.device(dev)` that costs nothing when `dev` is already the current device (the usual
+    case); kernels are launched on the current device, so the guard is needed only when it differs."""
+    __slots__ = ("guard",)
+
+    def __init__(self, dev: torch.device):
+        self.guard = None if dev.index is None or torch.cuda.current_device() == dev.index else torch.cuda.device(dev)
+
+    def __enter__(self):
+        if self.guard is not None:
+            self.guard.__enter__()
+
+    def __exit__(self, *exc):
+        if self.guard is not None:
+            return self.guard.__exit__(*exc)
+        return False
 
 
 def _rows(t: torch.Tensor) -> torch.Tensor:
@@ -101,7 +126,7 @@ def fused_swiglu_fwd(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, 
     out = torch.empty(out_shape, device=dev, dtype=dtype)
     g = torch.empty_like(out) if save_preactivations else None
     u = torch.empty_like(out) if save_preactivations else None
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         _abi.check(_abi.lib().fsw_swiglu_forward(
             x2.data_ptr(), wg.data_ptr(), wu.data_ptr(), out.data_ptr(),
             g.data_ptr() if g is not None else None, u.data_ptr() if u is not None else None,
@@ -122,7 +147,7 @@ def elementwise_backward(grad_output: torch.Tensor, xw_gate: torch.Tensor, xw_up
     dout, g, u = grad_output.contiguous(), xw_gate.contiguous(), xw_up.contiguous()
     grad_xw_up = torch.empty_like(dout)
     grad_xw_gate = torch.empty_like(dout)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         _abi.check(_abi.lib().fsw_elementwise_backward(
             dout.data_ptr(), g.data_ptr(), u.data_ptr(), grad_xw_up.data_ptr(),
             grad_xw_gate.data_ptr(), dout.numel(), _DTYPE_CODE[dtype], _stream_ptr(dev)))
@@ -153,7 +178,7 @@ def gating_grad_recompute(grad_output: torch.Tensor, x: torch.Tensor, w_gate: to
     dout = grad_output.contiguous()
     grad_xw_up = torch.empty_like(dout)
     grad_xw_gate = torch.empty_like(dout)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         _abi.check(_abi.lib().fsw_gating_grad_recompute(
             x2.data_ptr(), wg.data_ptr(), wu.data_ptr(), dout.data_ptr(), grad_xw_up.data_ptr(),
             grad_xw_gate.data_ptr(), x2.shape[0], D, I, _ld(x2), _ld(wg), I, _code(dtype, weights_out_in),
@@ -179,7 +204,7 @@ def fused_input_grad(grad_xw_gate: torch.Tensor, grad_xw_up: torch.Tensor, w_gat
         wg, wu = wg.contiguous(), wu.contiguous()
     T = dg.shape[0]
     grad_x = torch.empty(tuple(grad_xw_gate.shape[:-1]) + (D,), device=dev, dtype=dtype)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         flag = _abi.WEIGHTS_OUT_IN if weights_out_in else 0
         ws, ws_bytes = _workspace(_abi.STEP_INPUT_GRAD | flag, T, D, I, dev)
         _abi.check(_abi.lib().fsw_input_grad(
@@ -221,7 +246,7 @@ def fused_weight_grad(x: torch.Tensor, grad_xw_up: torch.Tensor, grad_xw_gate: t
         _require(grad_w_up.stride(-1) == 1 and grad_w_gate.stride(-1) == 1 and _ld(grad_w_up) == _ld(grad_w_gate)
                  and _ld(grad_w_up) >= wshape[1],
                  "weight-gradient outputs need unit inner stride and equal row strides")
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         flag = _abi.WEIGHTS_OUT_IN if weights_out_in else 0
         ws, ws_bytes = _workspace(_abi.STEP_WEIGHT_GRAD | flag, T, D, I, dev)
         _abi.check(_abi.lib().fsw_weight_grad(
@@ -249,7 +274,7 @@ def down_proj_forward(act: torch.Tensor, w_down: torch.Tensor, dtype: torch.dtyp
     T = a2.shape[0]
     y = torch.empty(tuple(act.shape[:-1]) + (D,), device=dev, dtype=dtype)
     flag = _abi.WEIGHTS_OUT_IN if weights_out_in else 0
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         ws, ws_bytes = _workspace(_abi.STEP_DOWN_FORWARD | flag, T, D, I, dev)
         _abi.check(_abi.lib().fsw_down_proj_forward(
             a2.data_ptr(), w2.data_ptr(), y.data_ptr(), T, I, D, _ld(a2), _ld(w2), D,
@@ -268,7 +293,7 @@ def down_proj_input_grad(grad_y: torch.Tensor, w_down: torch.Tensor, dtype: torc
     T = g2.shape[0]
     grad_act = torch.empty(tuple(grad_y.shape[:-1]) + (I,), device=dev, dtype=dtype)
     flag = _abi.WEIGHTS_OUT_IN if weights_out_in else 0
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         ws, ws_bytes = _workspace(_abi.STEP_DOWN_INPUT_GRAD | flag, T, D, I, dev)
         _abi.check(_abi.lib().fsw_down_proj_input_grad(
             g2.data_ptr(), w2.data_ptr(), grad_act.data_ptr(), T, I, D, _ld(g2), _ld(w2), I,
@@ -287,7 +312,7 @@ def down_proj_weight_grad(act: torch.Tensor, grad_y: torch.Tensor, dtype: torch.
     D = g2.shape[1]
     grad_w = torch.empty((D, I) if weights_out_in else (I, D), device=dev, dtype=dtype)
     flag = _abi.WEIGHTS_OUT_IN if weights_out_in else 0
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         ws, ws_bytes = _workspace(_abi.STEP_DOWN_WEIGHT_GRAD | flag, T, D, I, dev)
         _abi.check(_abi.lib().fsw_down_proj_weight_grad(
             a2.data_ptr(), g2.data_ptr(), grad_w.data_ptr(), T, I, D, _ld(a2), _ld(g2), grad_w.shape[1],
