@@ -155,7 +155,8 @@ def test_mlp_module_from_linear(oracle, dtype, keep_layout):
     assert oracle.rel_error(np64(y), np64(ref)) < 2 * tol
 
 
-FEW_TOKENS = [(1, 8, 8), (7, 72, 136), (16, 520, 392), (33, 1032, 136), (64, 200, 1160), (65, 64, 264), (128, 1096, 520)]
+FEW_TOKENS = [(1, 8, 8), (7, 72, 136), (16, 520, 392), (33, 1032, 136), (64, 200, 1160), (65, 64, 264), (128, 1096, 520),
+              (129, 264, 520), (256, 520, 392)]
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
@@ -163,15 +164,16 @@ FEW_TOKENS = [(1, 8, 8), (7, 72, 136), (16, 520, 392), (33, 1032, 136), (64, 200
 @pytest.mark.parametrize("tdi", FEW_TOKENS, ids=lambda s: "x".join(map(str, s)))
 def test_few_token_forward_in_both_layouts(oracle, dtype, out_in, tdi):
     """Up to 128 tokens the forward runs on the weight-streaming kernels (selection code 2), one per weight
-    layout: out and the saved pre-activations against the oracle, with reductions that are not multiples of a
-    stage (64 or 32 elements), ragged last column blocks and row counts on both sides of every variant."""
+    layout; up to 256 the tiled kernel has a single row of tiles and streams the weights past the caches: out and
+    the saved pre-activations against the oracle, with reductions that are not multiples of a stage (64
+    elements), ragged last column blocks and row counts on both sides of every variant."""
     T, D, I = tdi
     x, wg, wu, _, _, _ = make(oracle, (1, T, D, I), dtype, seed=T + D)
     tx = dev(x[0], dtype)
     twg, twu = (dev(wg.T, dtype), dev(wu.T, dtype)) if out_in else (dev(wg, dtype), dev(wu, dtype))
     ldw = D if out_in else I
     flag = _abi.WEIGHTS_OUT_IN if out_in else 0
-    assert _abi.lib().fsw_uses_tiled_kernel(flag, T, D, I, D, ldw, I, I, 16) == 2
+    assert _abi.lib().fsw_uses_tiled_kernel(flag, T, D, I, D, ldw, I, I, 16) == (2 if T <= 128 else 1)
     out, g, u = _launch.fused_swiglu_fwd(tx, twg, twu, dtype, weights_out_in=out_in)
     out_only = _launch.fused_swiglu_fwd(tx, twg, twu, dtype, save_preactivations=False, weights_out_in=out_in)[0]
     torch.cuda.synchronize()
