@@ -40,14 +40,16 @@ FSW_DEV i16x8 read_frag_kc32(const FSW_LDS char* area, int row_base, int ks, int
 }
 
 template <typename E, int BM, bool W_KC>
-__global__ __launch_bounds__(kSkThreads) void fsw_skinny_forward_kernel(GemmParams p) {
+__global__ __launch_bounds__(kSkThreads) void fsw_skinny_forward_kernel(GemmParams p, int bn) {
   using C = SkCfg<BM>;
   constexpr int NQ = BM / 32;
   constexpr int kStages = C::kStages, kStage = C::kStage, kXBytes = C::kXBytes;
   __shared__ __attribute__((aligned(1024))) char smem[kStages * kStage];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int n0 = blockIdx.x * 128;
+  // this workgroup's output columns n0 .. n0 + bn - 1 (bn <= 128: the rest of the 128-column slot stays
+  // out of range, costs no memory traffic and multiplies zeros)
+  const int n0 = blockIdx.x * bn;
   const int st_total = (p.K + 63) / 64;
   const unsigned smem_addr = (unsigned)(uintptr_t)(FSW_LDS char*)smem;
   const FSW_LDS char* smem_l = (const FSW_LDS char*)smem;
@@ -72,7 +74,7 @@ __global__ __launch_bounds__(kSkThreads) void fsw_skinny_forward_kernel(GemmPara
       const int c = (lane & 7) ^ ((row >> 1) & 7);
       const int n = row & 127;
       w_off[j] = (unsigned)n * (unsigned)p.ldb * 2u + c * 16u;
-      w_klim[j] = (n0 + n < p.N) ? p.K - c * 8 : -0x40000000;
+      w_klim[j] = (n < bn && n0 + n < p.N) ? p.K - c * 8 : -0x40000000;
       w_base[j] = (const char*)(j < 4 ? p.b0 : p.b1) + (size_t)n0 * p.ldb * 2;
     } else {
       // slot j >> 2 (k-rows 32*(j >> 2)..), instruction i = wave + 4*(j & 3) of its 16: panel i >> 3, 4 k-rows
@@ -80,7 +82,7 @@ __global__ __launch_bounds__(kSkThreads) void fsw_skinny_forward_kernel(GemmPara
       const int row = 32 * (j >> 2) + 4 * (i & 7) + (lane >> 4);
       const int col = (((lane >> 2) & 3) ^ ((lane >> 4) & 3)) * 32 + (lane & 3) * 8;
       w_off[j] = (unsigned)row * (unsigned)p.ldb * 2u + col * 2u;
-      w_klim[j] = (n0 + col < p.N) ? p.K - row : -0x40000000;
+      w_klim[j] = (col < bn && n0 + col < p.N) ? p.K - row : -0x40000000;
       w_base[j] = (const char*)((i >> 3) ? p.b1 : p.b0) + (size_t)n0 * 2;
     }
   }
@@ -161,8 +163,8 @@ __global__ __launch_bounds__(kSkThreads) void fsw_skinny_forward_kernel(GemmPara
     if (m >= p.M) continue;
 #pragma unroll
     for (int r4 = 0; r4 < 4; r4++) {
-      const int n = n0 + wave * 32 + 8 * r4 + 4 * (lane >> 5);
-      if (n >= p.N) continue;
+      const int nc = wave * 32 + 8 * r4 + 4 * (lane >> 5), n = n0 + nc;
+      if (nc >= bn || n >= p.N) continue;
       const size_t o = (size_t)m * p.ldc + n;
       unsigned short ho[4], hg[4], hu[4];
 #pragma unroll
@@ -189,12 +191,38 @@ __global__ __launch_bounds__(kSkThreads) void fsw_skinny_forward_kernel(GemmPara
 // kernel takes over.
 constexpr int kSkMaxRows = 128;
 
+// Width of a workgroup's column block.  128 columns fill the LDS slot, but a launch is one workgroup per block
+// and every block takes the same time, so what counts is rounds x width: the width that covers N with the
+// fewest rounds of `cus` workgroups wins (I = 28672 on 256 CUs: 256 blocks of 112 instead of 224 of 128;
+// I = 12288 and 16 rows: 256 blocks of 48 instead of 96 of 128).  Two limits, both measured:
+//  * weights stored [D, I] are read in row segments that must start on 128-byte lines (partial lines are
+//    fetched whole, by two workgroups): widths of 64 and 128 only; rows of [I, D] weights are lines of
+//    their own: any multiple of 8;
+//  * a narrower block leaves part of every 32 KiB weight slot empty while the x rows stay, so the useful
+//    bytes in flight per CU shrink: not below 48 / 64 / 96 columns for up to 32 / 64 / 128 rows.
+static int block_width(int N, int cus, bool w_kc, int bm) {
+  const int step = w_kc ? 8 : 64;
+  const int narrowest = w_kc ? (bm <= 32 ? 48 : (bm <= 64 ? 64 : 96)) : 64;
+  int best = 128;
+  long long best_cost = (long long)(((N + 127) / 128 + cus - 1) / cus) * 128;
+  for (int bn = 128 - step; bn >= narrowest; bn -= step) {
+    const long long cost = (long long)(((N + bn - 1) / bn + cus - 1) / cus) * bn;
+    if (cost < best_cost) { best = bn; best_cost = cost; }
+  }
+  return best;
+}
+
 template <typename E, bool W_KC>
 static hipError_t launch_skinny_t(const GemmParams& g, hipStream_t s) {
-  const unsigned tiles = (unsigned)((g.N + 127) / 128);
-  if (g.M <= 32) fsw_skinny_forward_kernel<E, 32, W_KC><<<tiles, kSkThreads, 0, s>>>(g);
-  else if (g.M <= 64) fsw_skinny_forward_kernel<E, 64, W_KC><<<tiles, kSkThreads, 0, s>>>(g);
-  else fsw_skinny_forward_kernel<E, 128, W_KC><<<tiles, kSkThreads, 0, s>>>(g);
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+    cus = 256;
+  const int bn = block_width(g.N, cus, W_KC, g.M);
+  const unsigned tiles = (unsigned)((g.N + bn - 1) / bn);
+  if (g.M <= 32) fsw_skinny_forward_kernel<E, 32, W_KC><<<tiles, kSkThreads, 0, s>>>(g, bn);
+  else if (g.M <= 64) fsw_skinny_forward_kernel<E, 64, W_KC><<<tiles, kSkThreads, 0, s>>>(g, bn);
+  else fsw_skinny_forward_kernel<E, 128, W_KC><<<tiles, kSkThreads, 0, s>>>(g, bn);
   return hipGetLastError();
 }
 
