@@ -321,7 +321,37 @@ def main():
                                     "peak_gbs": PEAK_HBM_GBS, "runs": skinny,
                                     "workload_weights_out_in": "the same with Wg/Wu stored [28672,8192] (nn.Linear layout)",
                                     "runs_weights_out_in": skinny_out_in}
-        del w_sets
+        # the down projection that follows, same model (y [M,8192] = act [M,28672] W_down), both storage orders
+        def down_runs(w_list, flag, ldw):
+            runs = []
+            scratch = torch.empty(int(L.fsw_workspace_bytes(_abi.STEP_DOWN_FORWARD | flag, 128, D4, I4)) or 16, device=dev, dtype=torch.uint8)
+            for M in (16, 64, 128):
+                act = torch.randn(M, I4, device=dev, dtype=dt)
+                y = torch.empty(M, D4, device=dev, dtype=dt)
+                state = {"i": 0}
+
+                def down():
+                    w = w_list[state["i"] % len(w_list)]
+                    state["i"] += 1
+                    _abi.check(L.fsw_down_proj_forward(p(act), p(w), p(y), M, I4, D4, I4, ldw, D4, p(scratch), scratch.numel(), flag, stream))
+
+                def vendor():
+                    w = w_list[state["i"] % len(w_list)]
+                    state["i"] += 1
+                    torch.matmul(act, w.t() if flag else w, out=y)
+
+                ms, ms_v = gpu_time_ms(down, iters=20), gpu_time_ms(vendor, iters=20)
+                nbytes = 2.0 * (D4 * I4 + M * I4 + M * D4)
+                runs.append({"M": M, "ms": round(ms, 4), "frac_hbm_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4),
+                             "vendor_ms": round(ms_v, 4), "vendor_frac_hbm_peak": round(nbytes / ms_v / 1e6 / PEAK_HBM_GBS, 4)})
+            return runs
+
+        flat = [w for pair in w_sets for w in pair]   # four arrays of D4*I4 elements, alternating: nothing stays cached
+        result["down_proj_few_tokens"] = {
+            "workload": "bf16 y [M,8192] = act [M,28672] W_down, W_down read once; vendor = torch.matmul on the same arrays",
+            "runs_w_down_DxI": down_runs([w.view(D4, I4) for w in flat], _abi.WEIGHTS_OUT_IN, I4),
+            "runs_w_down_IxD": down_runs([w.view(I4, D4) for w in flat], 0, D4)}
+        del w_sets, flat
 
     # ---- the other configurations, the eager PyTorch step and the vendor GEMMs on the same box
     if not args.no_extra:

@@ -3,6 +3,7 @@
 #include "fsw_internal.hpp"
 #include <cstdarg>
 #include <cstdio>
+#include <algorithm>
 #include <mutex>
 
 namespace {
@@ -95,8 +96,8 @@ int64_t fsw_workspace_bytes(int step, int64_t T, int64_t D, int64_t I) {
     case 1: return fsw::splitk_workspace_bytes(oi ? 4 : 1, T, D, I);
     case 2: return fsw::splitk_workspace_bytes(oi ? 5 : 2, T, D, I);
     // down projection: forward y [T,D] over I; input grad [T,I] over D; weight grad [I,D] ([D,I]) over T
-    case 4: return fsw::gemm_workspace_bytes(oi ? 1 : 0, T, D, I);
-    case 5: return fsw::gemm_workspace_bytes(oi ? 0 : 1, T, I, D);
+    case 4: return std::max(fsw::gemm_workspace_bytes(oi ? 1 : 0, T, D, I), fsw::skinny_gemm_workspace_bytes(oi ? 1 : 0, T, D, I));
+    case 5: return std::max(fsw::gemm_workspace_bytes(oi ? 0 : 1, T, I, D), fsw::skinny_gemm_workspace_bytes(oi ? 0 : 1, T, I, D));
     case 6: return oi ? fsw::gemm_workspace_bytes(2, D, I, T) : fsw::gemm_workspace_bytes(2, I, D, T);
     default: return 0;
   }
@@ -243,6 +244,8 @@ static int run_gemm(const char* fn, int layout, const void* a, const void* b, vo
   hipStream_t s = (hipStream_t)stream;
   if (fsw::fast_path_ok_gemm(p)) {
     const bool ws_ok = workspace && workspace_bytes > 0 && ((uintptr_t)workspace & 15) == 0;
+    if (fsw::skinny_gemm_ok(p))   // few rows: stream the weights
+      return launched(fn, fsw::launch_gemm_skinny(dtype, p, s, ws_ok ? workspace : nullptr, ws_ok ? workspace_bytes : 0));
     return launched(fn, fsw::launch_gemm_fast(dtype, p, s, ws_ok ? workspace : nullptr, ws_ok ? workspace_bytes : 0));
   }
   return launched(fn, fsw::launch_gemm_generic(dtype, p, s));

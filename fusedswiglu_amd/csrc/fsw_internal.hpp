@@ -51,6 +51,12 @@ long long splitk_workspace_bytes(int step, long long T, long long D, long long I
 bool skinny_forward_ok(const Problem& p);
 hipError_t launch_forward_skinny(int dtype, const Problem& p, hipStream_t s);
 
+// The same kernel as a plain GEMM for the down projection of few tokens (layouts 0 and 1, M <= 128, N even and
+// its half aligned); splits the reduction into the caller's scratch when column blocks alone leave CUs idle.
+bool skinny_gemm_ok(const GemmProblem& p);
+long long skinny_gemm_workspace_bytes(int layout, long long M, long long N, long long K);
+hipError_t launch_gemm_skinny(int dtype, const GemmProblem& p, hipStream_t s, void* ws, long long ws_bytes);
+
 // Any shape, any stride, 2-byte alignment: guarded element loads, same MFMA arithmetic.
 hipError_t launch_forward_generic(int dtype, const Problem& p, hipStream_t s);
 hipError_t launch_input_grad_generic(int dtype, const Problem& p, hipStream_t s);

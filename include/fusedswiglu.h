@@ -169,7 +169,10 @@ FSW_API int fsw_weight_grad(const void* x, const void* grad_xw_up, const void* g
  *   forward      y           = act W_down
  *   input_grad   grad_act    = grad_y W_down^T
  *   weight_grad  grad_w_down = act^T grad_y      (summed over all T tokens in fp32)
- * `workspace` as for fsw_input_grad (steps 4, 5, 6 of fsw_workspace_bytes).
+ * `workspace` as for fsw_input_grad (steps 4, 5, 6 of fsw_workspace_bytes).  Up to 128 tokens, forward and
+ * input_grad stream the weight once from HBM on the kernel of the few-token SwiGLU forward; the result is then
+ * short (D or I columns) and the reduction long, so the reduction is split over the CUs through `workspace`
+ * (without it the call is correct but leaves most CUs idle).
  */
 FSW_API int fsw_down_proj_forward(const void* act, const void* w_down, void* y, int64_t T, int64_t I, int64_t D,
                                   int64_t ld_act, int64_t ldw, int64_t ldy, void* workspace,

@@ -122,6 +122,40 @@ def test_down_projection_launchers(oracle, dtype, out_in, shape):
     assert oracle.rel_error(np64(d_w), o_dw.T if out_in else o_dw) < tol
 
 
+FEW_TOKENS_DOWN = [(1, 72, 128), (16, 520, 256), (33, 1096, 384), (64, 4104, 512), (100, 8200, 1024), (128, 2056, 1152)]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("out_in", [False, True], ids=["w_down_IxD", "w_down_DxI"])
+@pytest.mark.parametrize("tid", FEW_TOKENS_DOWN, ids=lambda s: "x".join(map(str, s)))
+def test_few_token_down_projection(oracle, dtype, out_in, tid):
+    """Up to 128 tokens the down projection (and its input gradient) streams the weights on the kernel of the
+    few-token forward, as a plain GEMM over the two column halves of W_down with the reduction split into the
+    caller's scratch: against the oracle with scratch (the launcher asks the library for it), and through the
+    raw ABI without scratch (no split), which must agree to within the rounding of one more fp32 summation order."""
+    T, I, D = tid
+    rng = np.random.default_rng(T + I)
+    rnd = oracle.rounder(NAME[dtype])
+    act = rnd(rng.standard_normal((T, I)))
+    wd = rnd(rng.standard_normal((I, D)) / I ** 0.5)
+    dy = rnd(rng.standard_normal((T, D)))
+    tact, tdy, twd = dev(act, dtype), dev(dy, dtype), dev(wd.T if out_in else wd, dtype)
+    y = _launch.down_proj_forward(tact, twd, dtype, weights_out_in=out_in)
+    d_act = _launch.down_proj_input_grad(tdy, twd, dtype, weights_out_in=out_in)
+    y_nosplit = torch.empty_like(y)
+    L, p = _abi.lib(), lambda t: t.data_ptr()
+    code = (_abi.DTYPE_BF16 if dtype == torch.bfloat16 else _abi.DTYPE_FP16) | (_abi.WEIGHTS_OUT_IN if out_in else 0)
+    _abi.check(L.fsw_down_proj_forward(p(tact), p(twd), p(y_nosplit), T, I, D, I, twd.shape[1], D, None, 0, code,
+                                       torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    o_da, _ = oracle.down_proj_backward(act, wd, dy)
+    tol = TOL[dtype]
+    assert oracle.rel_error(np64(y), oracle.down_proj_fwd(act, wd)) < tol
+    assert oracle.rel_error(np64(y_nosplit), oracle.down_proj_fwd(act, wd)) < tol
+    assert oracle.rel_error(np64(y), np64(y_nosplit)) < tol / 2
+    assert oracle.rel_error(np64(d_act), o_da) < tol
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 @pytest.mark.parametrize("keep_layout", [True, False], ids=["linear_layout", "reference_layout"])
 def test_mlp_module_from_linear(oracle, dtype, keep_layout):
