@@ -218,6 +218,35 @@ def test_few_token_forward_in_both_layouts(oracle, dtype, out_in, tdi):
     assert torch.equal(out, out_only)
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_few_token_random_shapes(oracle, seed):
+    """Seeded random few-token problems (T <= 128, dimensions multiples of 8 so that the streaming kernels run):
+    SwiGLU forward in a random layout and element type, then the down projection in a random storage order,
+    each against the oracle."""
+    rng = np.random.default_rng(1000 + seed)
+    dtype = (torch.bfloat16, torch.float16)[seed & 1]
+    T = int(rng.integers(1, 129))
+    D = 8 * int(rng.integers(1, 160))
+    I = 16 * int(rng.integers(1, 200))       # the down projection needs I / 2 aligned as well
+    out_in, down_out_in = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+    rnd = oracle.rounder(NAME[dtype])
+    x = rnd(rng.standard_normal((T, D)))
+    wg, wu = rnd(rng.standard_normal((D, I)) / D ** 0.5), rnd(rng.standard_normal((D, I)) / D ** 0.5)
+    wd = rnd(rng.standard_normal((I, D)) / I ** 0.5)
+    tx = dev(x, dtype)
+    twg, twu = (dev(wg.T, dtype), dev(wu.T, dtype)) if out_in else (dev(wg, dtype), dev(wu, dtype))
+    out, g, u = _launch.fused_swiglu_fwd(tx, twg, twu, dtype, weights_out_in=out_in)
+    torch.cuda.synchronize()
+    o_out, o_g, o_u = oracle.fused_swiglu_fwd(x, wg, wu)
+    tol = TOL[dtype]
+    assert oracle.rel_error(np64(out), o_out) < tol, (T, D, I, out_in)
+    assert oracle.rel_error(np64(g), o_g) < tol and oracle.rel_error(np64(u), o_u) < tol
+    act = np64(out)
+    y = _launch.down_proj_forward(out, dev(wd.T if down_out_in else wd, dtype), dtype, weights_out_in=down_out_in)
+    torch.cuda.synchronize()
+    assert oracle.rel_error(np64(y), oracle.down_proj_fwd(act, wd)) < tol, (T, D, I, down_out_in)
+
+
 def test_linear_layout_full_size_forward_slices(oracle):
     """The headline shape with nn.Linear-layout weights: whole token rows of out against the oracle."""
     dtype, T, D, I = torch.bfloat16, 8192, 4096, 12288
