@@ -435,52 +435,59 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
     v.y = E::from_float(c) | ((unsigned)E::from_float(d) << 16);
     return v;
   };
+  if constexpr (C::kForward) {
+    // out = silu(g) * u, then g and u themselves (skipped when the caller passes no buffers for them); in
+    // gating-gradient mode (d0 given) dG and dU take the places of g and u and out is not written.  The mode is
+    // a compile-time parameter of the body so that the inner loops carry no branch on it.
+    auto forward_tile = [&](auto gating_tag) {
+      constexpr bool gating = decltype(gating_tag)::value;
 #pragma unroll
-  for (int q = 0; q < 2; q++) {  // 32 rows of the wave's 64 at a time
-    if constexpr (C::kForward) {
-      // gating-gradient mode: this lane's upstream gradients, 4 consecutive columns per 16x16 block
-      u32x2 dv[2][4];
-      const bool gating = p.d0 != nullptr;
-      if (gating) {
+      for (int q = 0; q < 2; q++) {  // 32 rows of the wave's 64 at a time
+        // gating-gradient mode: this lane's upstream gradients, 4 consecutive columns per 16x16 block
+        u32x2 dv[2][4];
+        if constexpr (gating) {
 #pragma unroll
-        for (int mbl = 0; mbl < 2; mbl++)
+          for (int mbl = 0; mbl < 2; mbl++)
 #pragma unroll
-          for (int c = 0; c < 4; c++) {
-            const int m = row_base + (2 * q + mbl) * 16 + (lane & 15);
-            const int n = n0 + wn * 64 + c * 16 + 4 * (lane >> 4);
-            dv[mbl][c] = (m < p.M && n < p.N) ? *(const u32x2*)((const unsigned short*)p.d0 + (size_t)m * p.ldc + n)
-                                              : u32x2{0u, 0u};
-          }
-      }
-      // out = silu(g) * u, then g and u themselves (skipped when the caller passes no buffers for them);
-      // in gating-gradient mode dG and dU take the places of g and u and out is not written
-#pragma unroll
-      for (int which = 0; which < 3; which++) {
-        if (which == 0 && gating) continue;
-        if (which > 0 && p.c1 == nullptr) break;
-#pragma unroll
-        for (int mbl = 0; mbl < 2; mbl++)
-#pragma unroll
-          for (int c = 0; c < 4; c++) {
-            const f32x4 g = acc[c][2 * q + mbl], u = acc[4 + c][2 * q + mbl];
-            float v[4];
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-              if (gating) {
-                const unsigned w = e < 2 ? dv[mbl][c].x : dv[mbl][c].y;
-                float dU, dG;
-                gating_grad(E::to_float((unsigned short)((e & 1) ? (w >> 16) : (w & 0xffffu))), g[e], u[e], dU, dG);
-                v[e] = which == 1 ? dG : dU;
-              } else {
-                v[e] = which == 0 ? silu_mul(g[e], u[e]) : (which == 1 ? g[e] : u[e]);
-              }
+            for (int c = 0; c < 4; c++) {
+              const int m = row_base + (2 * q + mbl) * 16 + (lane & 15);
+              const int n = n0 + wn * 64 + c * 16 + 4 * (lane >> 4);
+              dv[mbl][c] = (m < p.M && n < p.N) ? *(const u32x2*)((const unsigned short*)p.d0 + (size_t)m * p.ldc + n)
+                                                : u32x2{0u, 0u};
             }
-            *(FSW_LDS u32x2*)(patch + wr_off(mbl, c)) = pack4(v[0], v[1], v[2], v[3]);
-          }
-        unsigned short* dst = (unsigned short*)(which == 0 ? p.c0 : (which == 1 ? p.c1 : p.c2));
-        flush_patch(dst, n0 + wn * 64, q);
+        }
+#pragma unroll
+        for (int which = gating ? 1 : 0; which < 3; which++) {
+          if (which > 0 && p.c1 == nullptr) break;
+#pragma unroll
+          for (int mbl = 0; mbl < 2; mbl++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+              const f32x4 g = acc[c][2 * q + mbl], u = acc[4 + c][2 * q + mbl];
+              float v[4];
+#pragma unroll
+              for (int e = 0; e < 4; e++) {
+                if constexpr (gating) {
+                  const unsigned w = e < 2 ? dv[mbl][c].x : dv[mbl][c].y;
+                  float dU, dG;
+                  gating_grad(E::to_float((unsigned short)((e & 1) ? (w >> 16) : (w & 0xffffu))), g[e], u[e], dU, dG);
+                  v[e] = which == 1 ? dG : dU;
+                } else {
+                  v[e] = which == 0 ? silu_mul(g[e], u[e]) : (which == 1 ? g[e] : u[e]);
+                }
+              }
+              *(FSW_LDS u32x2*)(patch + wr_off(mbl, c)) = pack4(v[0], v[1], v[2], v[3]);
+            }
+          unsigned short* dst = (unsigned short*)(which == 0 ? p.c0 : (which == 1 ? p.c1 : p.c2));
+          flush_patch(dst, n0 + wn * 64, q);
+        }
       }
-    } else {
+    };
+    if (p.d0 != nullptr) forward_tile(std::true_type{});
+    else forward_tile(std::false_type{});
+  } else {
+#pragma unroll
+    for (int q = 0; q < 2; q++) {  // 32 rows of the wave's 64 at a time
 #pragma unroll
       for (int h = 0; h < 2; h++) {  // the wave's two groups of 64 columns
 #pragma unroll
