@@ -135,7 +135,7 @@ FSW_DEV void wait_vmcnt_and_barrier() {
 //   (the tiled kernel additionally swaps the 32-byte halves of every block on k-rows 8..15 and
 //   24..31, see read_frag_mc16).
 // The k-contiguous formats (rows of 128 or 64 bytes with XOR-swizzled 16-byte chunks) are described
-// where they are read: read_frag_kc in fsw_gemm.hpp, read_frag_x in fsw_skinny.hip.
+// where they are read: read_frag_kc16 in fsw_gemm.hpp, read_frag_kc32 in fsw_skinny.hip.
 constexpr int kBK = 32;
 constexpr int kMcRowBytes = 256;
 constexpr int kMcPanelBytes = kBK * kMcRowBytes;  // 8 KiB
