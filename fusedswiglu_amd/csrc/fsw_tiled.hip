@@ -1,5 +1,7 @@
 // Host side of the tiled MFMA kernels: eligibility checks and launches.
 #include "fsw_gemm.hpp"
+#include "fsw_gemm4.hpp"
+#include <cstdlib>
 #include "fsw_internal.hpp"
 
 namespace fsw {
@@ -119,6 +121,29 @@ static hipError_t launch(int dtype, GemmParams g, hipStream_t s, void* ws = null
   g.ws = (float*)ws; g.splits = pl.splits; g.steps_per_split = pl.steps_per_split;
   const long long grid = tiles * pl.splits;
   if (grid > 0x7fffffffLL) return hipErrorInvalidValue;
+  static const int w4_mask_env = getenv("FSW_W4") ? atoi(getenv("FSW_W4")) : 0;
+  // the four-wave kernel walks an m/n-contiguous operand through 32-bit offsets from its first k-row
+  const bool w4_fits = (Cfg<MODE>::kAKc || (long long)g.K * g.lda * 2 < (1LL << 31)) &&
+                       (Cfg<MODE>::kBKc || (long long)g.K * g.ldb * 2 < (1LL << 31));
+  const int w4_mask = w4_fits ? w4_mask_env : 0;
+#ifdef FSW_DEV_FAST
+  if (MODE <= 2 && ((w4_mask >> MODE) & 1)) {
+    if constexpr (MODE <= 2)
+#else
+  if ((w4_mask >> MODE) & 1) {
+#endif
+#ifdef FSW_DEV_FAST
+    fsw_gemm4_kernel<BF16, MODE><<<(unsigned)grid, kThreads4, 0, s>>>(g);
+#else
+    if (Cfg<MODE>::kForward && g.tiles_m == 1) {
+      if constexpr (Cfg<MODE>::kForward) {
+        if (dtype == kDtypeBF16) fsw_gemm4_kernel<BF16, MODE, true><<<(unsigned)grid, kThreads4, 0, s>>>(g);
+        else fsw_gemm4_kernel<FP16, MODE, true><<<(unsigned)grid, kThreads4, 0, s>>>(g);
+      }
+    } else if (dtype == kDtypeBF16) fsw_gemm4_kernel<BF16, MODE><<<(unsigned)grid, kThreads4, 0, s>>>(g);
+    else fsw_gemm4_kernel<FP16, MODE><<<(unsigned)grid, kThreads4, 0, s>>>(g);
+#endif
+  } else
   // a forward with a single row of tiles reads every weight byte exactly once: stream them past the caches
   if (Cfg<MODE>::kForward && g.tiles_m == 1) {
     if constexpr (Cfg<MODE>::kForward) {
