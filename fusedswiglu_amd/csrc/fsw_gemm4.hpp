@@ -8,14 +8,19 @@
 //
 // With a single wave per SIMD nothing hides a bubble in that wave's instruction stream, so the main loop is
 // written out MFMA by MFMA: after each of the 128 MFMAs of a pair of steps there is one "gap" that holds at
-// most a few other instructions (one fragment read, or one half of a direct-to-LDS load), and nothing is
-// allowed to move between gaps.  Per pair p (steps 2p and 2p+1, fragment register sets 0 and 1):
-//   gaps   0.. 31   the 8 loads of A(p+2) (ring slot of pair p-1, released at the last barrier)
-//   gaps  32.. 63   fragment reads of step 2p+1 into set 1
-//   gap   72        s_waitcnt vmcnt(8) lgkmcnt(0); s_barrier: pair p+1 has landed for every wave, and every
+// most a few other instructions, and nothing is allowed to move between gaps.  What a gap can hold for free was
+// measured with one wave per SIMD issuing 16x16x32 MFMAs back to back (16 cycles each): one scalar instruction
+// (every further one costs 8 cycles), two vector ALU instructions, one LDS read (two behind the same MFMA cost
+// 17 cycles), or one direct-to-LDS load (about 12 cycles in any case).  Per pair p (steps 2p and 2p+1, fragment
+// register sets 0 and 1):
+//   gaps   0.. 14   the A stream moves on to pair p+2, one or two scalar instructions per gap
+//   gaps  15.. 58   the 8 loads of A(p+2) (ring slot of pair p-1, released at the last barrier), one per 6 gaps
+//   gaps  16.. 47   fragment reads of step 2p+1 into set 1, one LDS instruction per gap
+//   gaps  46.. 60   the B stream moves on to pair p+2
+//   gap   64        s_waitcnt vmcnt(8) lgkmcnt(0); s_barrier: pair p+1 has landed for every wave, and every
 //                   wave has finished reading pair p out of LDS
-//   gaps  74..105   the 8 loads of B(p+2) into pair p's B space
-//   gaps  96..127   fragment reads of step 2p+2 into set 0
+//   gaps  66..109   the 8 loads of B(p+2) into pair p's B space
+//   gaps  80..111   fragment reads of step 2p+2 into set 0
 #pragma once
 #include <utility>
 
@@ -24,9 +29,6 @@
 namespace fsw {
 
 constexpr int kThreads4 = 256;
-#ifndef FSW4_OPT
-#define FSW4_OPT 0
-#endif
 // index i (0 <= i < count) with start + stride*i == g, or -1
 constexpr int gap_index(int g, int start, int stride, int count) {
   return (g >= start && (g - start) % stride == 0 && (g - start) / stride < count) ? (g - start) / stride : -1;
@@ -261,7 +263,6 @@ __global__ __launch_bounds__(kThreads4) void fsw_gemm4_kernel(GemmParams p) {
   // offset; the load itself comes at least one instruction later (M0 write -> LDS-DMA use).
   auto load_prep = [&](const Stream4& S, const Loader4& L, bool kc, int i) -> unsigned {
     asm volatile("s_add_u32 m0, %0, %1" : : "s"(S.dst), "n"(i * 4096) : "scc", "memory");
-    if ((FSW4_OPT & 8) != 0) return kOobOffset;
     // the whole offset goes through the vector operand, which the descriptor's range check covers for certain
     if (kc) return S.ok[0] ? L.voff[i] + S.koff : kOobOffset;
     return S.ok[(i >> 2) * 2 + (i & 1)] ? L.voff[i & 3] + S.soff[i >> 2] : kOobOffset;
@@ -352,16 +353,16 @@ __global__ __launch_bounds__(kThreads4) void fsw_gemm4_kernel(GemmParams p) {
 
   // The schedule of one pair: which gap (after MFMA g of 128) holds what.
   //   kAMicro0 + n                 micro-step n of moving the A stream on to pair p+2
-  //   kALd0 + kLdStride*i, +1      preparation and issue of load i of A(p+2)
+  //   kALd0 + kLdStrideA*i, +1     preparation and issue of load i of A(p+2)
   //   kRd1_0 + r                   read slot r of step 2p+1 (set 1)
   //   kBMicro0 + n, kBarrier       the B stream moves on to pair p+2; the barrier of pair p
-  //   kBLd0 + kLdStride*i, +1      loads of B(p+2), after the barrier
+  //   kBLd0 + kLdStrideB*i, +1     loads of B(p+2), after the barrier
   //   kRdNext .. +3                the ring offsets of pair p+1
   //   kRd0_0 + r                   read slot r of step 2p+2 (set 0), after the barrier
-  constexpr int kLdStride = 6;
+  constexpr int kLdStrideA = 6, kLdStrideB = 6;
   constexpr int kAMicro0 = 0, kALd0 = 15, kRd1_0 = 16;
   constexpr int kBMicro0 = 46, kBarrier = 64, kBLd0 = 66, kRdNext = 74, kRd0_0 = 80;
-  static_assert(kALd0 + 1 + 7 * kLdStride < kBarrier && kBLd0 > kBarrier && kBLd0 + 1 + 7 * kLdStride < 128, "load gaps");
+  static_assert(kALd0 + 1 + 7 * kLdStrideA < kBarrier && kBLd0 > kBarrier && kBLd0 + 1 + 7 * kLdStrideB < 128, "load gaps");
   static_assert(kRd1_0 + 31 < kBarrier && kRd0_0 > kBarrier && kRd0_0 + 31 < 128, "read gaps");
 
   for (int kt = 0; kt < kt_total; kt += 2) {
@@ -376,26 +377,22 @@ __global__ __launch_bounds__(kThreads4) void fsw_gemm4_kernel(GemmParams p) {
       // --- the A stream moves on to pair p+2 (ring slot of pair p-1, released at the last barrier); its loads
       if constexpr (g >= kAMicro0 && g < kAMicro0 + 15)
         stream_micro(sa, la, A_KC, smem_a, C::kPairsA, wrap_a0, wrap_a1, g - kAMicro0);
-      constexpr int ia_prep = gap_index(g, kALd0, kLdStride, 8), ia_go = gap_index(g, kALd0 + 1, kLdStride, 8);
-      if constexpr (!(FSW4_OPT & 1)) {
-        if constexpr (ia_prep >= 0) off_a = load_prep(sa, la, A_KC, ia_prep);
-        if constexpr (ia_go >= 0) load_go(sa, la, A_KC, false, ia_go, off_a, keep);
-      }
+      constexpr int ia_prep = gap_index(g, kALd0, kLdStrideA, 8), ia_go = gap_index(g, kALd0 + 1, kLdStrideA, 8);
+      if constexpr (ia_prep >= 0) off_a = load_prep(sa, la, A_KC, ia_prep);
+      if constexpr (ia_go >= 0) load_go(sa, la, A_KC, false, ia_go, off_a, keep);
       // --- fragments of step kt+1 (second half of the same pair) into set 1
       if constexpr (g == kRd1_0 - 1) {
         ra = lds0 + rd_pair_a + rd_a[1];
         rb = lds0 + C::kBytesA + rd_pair_b + rd_b[1];
       }
-      if constexpr (!(FSW4_OPT & 4)) if constexpr (g >= kRd1_0 && g < kRd1_0 + 32) read_slot(1, g - kRd1_0, ra, rb);
+      if constexpr (g >= kRd1_0 && g < kRd1_0 + 32) read_slot(1, g - kRd1_0, ra, rb);
       // --- the B stream moves on to pair p+2; the barrier of pair p; the loads of B(p+2) into pair p's space
       if constexpr (g >= kBMicro0 && g < kBMicro0 + 15)
         stream_micro(sb, lb, B_KC, smem_b, C::kPairsB, wrap_b0, wrap_b1, g - kBMicro0);
-      if constexpr (!(FSW4_OPT & 2)) if constexpr (g == kBarrier) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-      constexpr int ib_prep = gap_index(g, kBLd0, kLdStride, 8), ib_go = gap_index(g, kBLd0 + 1, kLdStride, 8);
-      if constexpr (!(FSW4_OPT & 1)) {
-        if constexpr (ib_prep >= 0) off_b = load_prep(sb, lb, B_KC, ib_prep);
-        if constexpr (ib_go >= 0) load_go(sb, lb, B_KC, B_INTER, ib_go, off_b, hint_b);
-      }
+      if constexpr (g == kBarrier) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      constexpr int ib_prep = gap_index(g, kBLd0, kLdStrideB, 8), ib_go = gap_index(g, kBLd0 + 1, kLdStrideB, 8);
+      if constexpr (ib_prep >= 0) off_b = load_prep(sb, lb, B_KC, ib_prep);
+      if constexpr (ib_go >= 0) load_go(sb, lb, B_KC, B_INTER, ib_go, off_b, hint_b);
       // --- fragments of step kt+2 (pair p+1) into set 0
       if constexpr (g == kRdNext) { FSW_PIN_S(rd_pair_a); rd_pair_a += kKcAreaBytes; FSW_PIN_S(rd_pair_a); }
       if constexpr (g == kRdNext + 1) { FSW_PIN_S(rd_pair_a); rd_pair_a = rd_pair_a == C::kPairsA * kKcAreaBytes ? 0u : rd_pair_a; FSW_PIN_S(rd_pair_a); }
@@ -404,7 +401,7 @@ __global__ __launch_bounds__(kThreads4) void fsw_gemm4_kernel(GemmParams p) {
         ra = lds0 + rd_pair_a + rd_a[0];
         rb = lds0 + C::kBytesA + rd_pair_b + rd_b[0];
       }
-      if constexpr (!(FSW4_OPT & 4)) if constexpr (g >= kRd0_0 && g < kRd0_0 + 32) read_slot(0, g - kRd0_0, ra, rb);
+      if constexpr (g >= kRd0_0 && g < kRd0_0 + 32) read_slot(0, g - kRd0_0, ra, rb);
       __builtin_amdgcn_sched_barrier(0);
     });
   }

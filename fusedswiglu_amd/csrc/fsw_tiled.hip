@@ -1,7 +1,6 @@
 // Host side of the tiled MFMA kernels: eligibility checks and launches.
 #include "fsw_gemm.hpp"
 #include "fsw_gemm4.hpp"
-#include <cstdlib>
 #include "fsw_internal.hpp"
 
 namespace fsw {
@@ -121,20 +120,19 @@ static hipError_t launch(int dtype, GemmParams g, hipStream_t s, void* ws = null
   g.ws = (float*)ws; g.splits = pl.splits; g.steps_per_split = pl.steps_per_split;
   const long long grid = tiles * pl.splits;
   if (grid > 0x7fffffffLL) return hipErrorInvalidValue;
-  static const int w4_mask_env = getenv("FSW_W4") ? atoi(getenv("FSW_W4")) : 0;
-  // the four-wave kernel walks an m/n-contiguous operand through 32-bit offsets from its first k-row
+  // Which form of the kernel: four waves with 128 x 128 wave tiles read a third less from LDS per MFMA and run
+  // the long reductions 3-8 % faster; their prologue and epilogue are slower (half the waves), so short reductions
+  // stay on the eight-wave form (measured cross-over: about 64 steps, 96 for the forwards with their three
+  // results).  The four-wave form walks an m/n-contiguous operand through 32-bit offsets from its first k-row.
   const bool w4_fits = (Cfg<MODE>::kAKc || (long long)g.K * g.lda * 2 < (1LL << 31)) &&
                        (Cfg<MODE>::kBKc || (long long)g.K * g.ldb * 2 < (1LL << 31));
-  const int w4_mask = w4_fits ? w4_mask_env : 0;
-#ifdef FSW_DEV_FAST
-  if (MODE <= 2 && ((w4_mask >> MODE) & 1)) {
-    if constexpr (MODE <= 2)
+  const int steps_per_workgroup = pl.splits > 1 ? pl.steps_per_split : steps;
+#if defined(FSW_FORCE_WAVES)
+  const bool four_waves = w4_fits && FSW_FORCE_WAVES == 4;
 #else
-  if ((w4_mask >> MODE) & 1) {
+  const bool four_waves = w4_fits && steps_per_workgroup >= (Cfg<MODE>::kForward ? 96 : 64);
 #endif
-#ifdef FSW_DEV_FAST
-    fsw_gemm4_kernel<BF16, MODE><<<(unsigned)grid, kThreads4, 0, s>>>(g);
-#else
+  if (four_waves) {
     if (Cfg<MODE>::kForward && g.tiles_m == 1) {
       if constexpr (Cfg<MODE>::kForward) {
         if (dtype == kDtypeBF16) fsw_gemm4_kernel<BF16, MODE, true><<<(unsigned)grid, kThreads4, 0, s>>>(g);
@@ -142,7 +140,6 @@ static hipError_t launch(int dtype, GemmParams g, hipStream_t s, void* ws = null
       }
     } else if (dtype == kDtypeBF16) fsw_gemm4_kernel<BF16, MODE><<<(unsigned)grid, kThreads4, 0, s>>>(g);
     else fsw_gemm4_kernel<FP16, MODE><<<(unsigned)grid, kThreads4, 0, s>>>(g);
-#endif
   } else
   // a forward with a single row of tiles reads every weight byte exactly once: stream them past the caches
   if (Cfg<MODE>::kForward && g.tiles_m == 1) {
