@@ -54,7 +54,13 @@ struct GemmParams {
   // to c0/c1.
   float* ws;
   int splits, steps_per_split;
+  // tail split (four-wave kernel, every mode but the forwards, splits == 1): the tiles of the last, partial round
+  // of 256 workgroups - launch indices tail_first .. tail_first + tail_count - 1 - are each given to tail_parts
+  // workgroups that reduce tail_steps steps (even) and leave an fp32 partial tile in ws[tile][part][kTileFloats];
+  // fsw_tail_reduce_kernel adds the parts in a fixed order.  tail_count == 0: off.
+  int tail_first, tail_count, tail_parts, tail_steps;
 };
+constexpr int kTileFloats = 256 * 256;  // accumulators of one workgroup
 
 constexpr int kThreads = 512;
 constexpr int kMcSlotBytes = 2 * kMcPanelBytes;  // two 128-column panels: 16 KiB

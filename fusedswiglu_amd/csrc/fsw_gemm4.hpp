@@ -140,16 +140,21 @@ __global__ __launch_bounds__(kThreads4) void fsw_gemm4_kernel(GemmParams p) {
   const int wm = wave >> 1, wn = wave & 1;  // 2 waves along M x 2 along N
 
   const int ntiles = p.tiles_m * p.tiles_n;
-  const int split = C::kForward ? 0 : (int)(blockIdx.x / ntiles);
-  const TileCoord tc = xcd_tile_order((int)(blockIdx.x - split * ntiles), p.tiles_m, p.tiles_n, p.group_m);
+  // a workgroup of the tail split: part `tail_part` of the tile with launch index tail_first + tail_tile
+  const bool in_tail = !C::kForward && p.tail_count > 0 && (int)blockIdx.x >= p.tail_first;
+  const int tail_part = in_tail ? ((int)blockIdx.x - p.tail_first) / p.tail_count : 0;
+  const int tail_tile = in_tail ? ((int)blockIdx.x - p.tail_first) % p.tail_count : 0;
+  const int split = (C::kForward || in_tail) ? 0 : (int)(blockIdx.x / ntiles);
+  const int tile_index = in_tail ? p.tail_first + tail_tile : (int)(blockIdx.x - split * ntiles);
+  const TileCoord tc = xcd_tile_order(tile_index, p.tiles_m, p.tiles_n, p.group_m);
   const int m0 = tc.tm * TM;
   const int n0 = tc.tn * TN;
 
   // steps per pass; the two-pass modes (dG.W then dU.W) keep pairs of steps inside a pass
   const int kt1 = (C::kPasses == 2) ? (((p.K + kBK - 1) / kBK + 1) & ~1) : (p.K + kBK - 1) / kBK;
   const int kt_all = C::kPasses * kt1;
-  const int kbase = split * p.steps_per_split;
-  const int kt_total = C::kForward ? kt_all : min(p.steps_per_split, kt_all - kbase);
+  const int kbase = in_tail ? tail_part * p.tail_steps : split * p.steps_per_split;
+  const int kt_total = C::kForward ? kt_all : min(in_tail ? p.tail_steps : p.steps_per_split, kt_all - kbase);
 
   const unsigned smem_a = (unsigned)(uintptr_t)(FSW_LDS char*)smem;
   const unsigned smem_b = smem_a + C::kBytesA;
@@ -428,6 +433,20 @@ __global__ __launch_bounds__(kThreads4) void fsw_gemm4_kernel(GemmParams p) {
     else if constexpr (C::kDualM) return wm;
     else return 0;
   };
+  if (in_tail) {
+    // fp32 partial tile in tile-local coordinates [result][row][column], 16 bytes per lane and store
+    float* part = p.ws + ((size_t)tail_tile * p.tail_parts + tail_part) * kTileFloats;
+#pragma unroll
+    for (int mb = 0; mb < 8; mb++) {
+      const int r = row_base - m0 + mb * 16 + (lane & 15);
+#pragma unroll
+      for (int nb = 0; nb < 8; nb++) {
+        const int c = col_of_half(nb >> 2) - n0 + (nb & 3) * 16 + 4 * (lane >> 4);
+        *(f32x4*)(part + ((size_t)result_of_half(nb >> 2) * TM + r) * TN + c) = acc[nb][mb];
+      }
+    }
+    return;
+  }
   if (!C::kForward && p.splits > 1) {
     const size_t plane = (size_t)p.M * p.N;
 #pragma unroll
@@ -532,6 +551,33 @@ __global__ __launch_bounds__(kThreads4) void fsw_gemm4_kernel(GemmParams p) {
         flush_patch((unsigned short*)(result_of_half(h) == 0 ? p.c0 : p.c1), col_of_half(h), q);
       }
     }
+  }
+}
+
+// Results of the tail tiles: out[tile] = round(sum over parts of ws[tile][part]), fixed order.  One workgroup of
+// 256 threads per 32 rows x 256 floats of a tile (blockIdx.y = tail tile, blockIdx.x = slice of its 2*TM*TN / 8192).
+template <typename E, int MODE>
+__global__ __launch_bounds__(256) void fsw_tail_reduce_kernel(GemmParams p) {
+  using C = Cfg<MODE>;
+  constexpr int TM = C::kTileM, TN = C::kTileN;
+  const TileCoord tc = xcd_tile_order(p.tail_first + (int)blockIdx.y, p.tiles_m, p.tiles_n, p.group_m);
+  const float* ws = p.ws + (size_t)blockIdx.y * p.tail_parts * kTileFloats;
+#pragma unroll
+  for (int it = 0; it < 8; it++) {
+    const int i4 = ((int)blockIdx.x * 2048 + it * 256 + (int)threadIdx.x) * 4;  // float index in the tile
+    f32x4 a = *(const f32x4*)(ws + i4);
+    for (int s = 1; s < p.tail_parts; s++) {
+      const f32x4 b = *(const f32x4*)(ws + (size_t)s * kTileFloats + i4);
+      a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+    }
+    const int which = i4 / (TM * TN), rem = i4 - which * (TM * TN);
+    const int m = tc.tm * TM + rem / TN, n = tc.tn * TN + rem % TN;
+    if (m >= p.M || n >= p.N) continue;
+    u32x2 v;
+    v.x = E::from_float(a.x) | ((unsigned)E::from_float(a.y) << 16);
+    v.y = E::from_float(a.z) | ((unsigned)E::from_float(a.w) << 16);
+    unsigned short* out = (unsigned short*)(which == 0 ? p.c0 : p.c1);
+    *(u32x2*)(out + (size_t)m * p.ldc + n) = v;
   }
 }
 

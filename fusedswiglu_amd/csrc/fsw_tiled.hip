@@ -70,6 +70,28 @@ static SplitPlan plan_split(long long tiles, int steps, long long M, long long N
   if (pl.splits > 1 && (!ws || (long long)pl.splits * M * N * 4 * results > ws_bytes)) return SplitPlan{1, steps};
   return pl;
 }
+// Tail split: when the tiles do not fill the last round of 256 workgroups, each tile of that round goes to
+// `parts` workgroups that reduce a slice each (fsw_gemm.hpp, GemmParams).  Only for long reductions and at
+// least one full round before; the partial tiles take count * parts * 256 KiB of scratch.
+struct TailPlan { int first, count, parts, steps; };
+static TailPlan plan_tail(long long tiles, int steps) {
+  TailPlan t{0, 0, 1, steps};
+  const int count = (int)(tiles % 256);
+  if (tiles < 256 || count == 0 || count > 128 || steps < 128) return t;
+  int parts = 256 / count;
+  if (parts > 8) parts = 8;
+  if (parts > steps / 32) parts = steps / 32;
+  if (parts < 2) return t;
+  int sp = (steps + parts - 1) / parts;
+  sp = (sp + 1) & ~1;  // pairs of steps stay together
+  t.first = (int)(tiles - count);
+  t.count = count;
+  t.steps = sp;
+  t.parts = (steps + sp - 1) / sp;
+  return t;
+}
+static long long tail_bytes(const TailPlan& t) { return (long long)t.count * t.parts * kTileFloats * 4; }
+
 static int steps_of(int mode, long long K) {
   int steps = (int)((K + kBK - 1) / kBK);
   return (mode == kDx || mode == kDxT) ? 2 * ((steps + 1) & ~1) : steps;
@@ -81,7 +103,8 @@ static long long workspace_of(long long M, long long N, long long K) {
   using C = Cfg<MODE>;
   const long long tiles = ((M + C::kTileM - 1) / C::kTileM) * ((N + C::kTileN - 1) / C::kTileN);
   const SplitPlan pl = plan_split_unbounded(tiles, steps_of(MODE, K), M, N, C::kResults);
-  return pl.splits > 1 ? (long long)pl.splits * M * N * 4 * C::kResults : 0;
+  if (pl.splits > 1) return (long long)pl.splits * M * N * 4 * C::kResults;
+  return tail_bytes(plan_tail(tiles, steps_of(MODE, K)));
 }
 
 long long splitk_workspace_bytes(int step, long long T, long long D, long long I) {
@@ -132,7 +155,16 @@ static hipError_t launch(int dtype, GemmParams g, hipStream_t s, void* ws = null
 #else
   const bool four_waves = w4_fits && steps_per_workgroup >= (Cfg<MODE>::kForward ? 96 : 64);
 #endif
+  long long grid4 = grid;
+  if constexpr (!Cfg<MODE>::kForward) {
+    const TailPlan tp = plan_tail(tiles, steps);
+    if (four_waves && pl.splits == 1 && tp.count > 0 && ws && tail_bytes(tp) <= ws_bytes) {
+      g.tail_first = tp.first; g.tail_count = tp.count; g.tail_parts = tp.parts; g.tail_steps = tp.steps;
+      grid4 = tp.first + (long long)tp.count * tp.parts;
+    }
+  }
   if (four_waves) {
+    const long long grid = grid4;
     if (Cfg<MODE>::kForward && g.tiles_m == 1) {
       if constexpr (Cfg<MODE>::kForward) {
         if (dtype == kDtypeBF16) fsw_gemm4_kernel<BF16, MODE, true><<<(unsigned)grid, kThreads4, 0, s>>>(g);
@@ -150,7 +182,16 @@ static hipError_t launch(int dtype, GemmParams g, hipStream_t s, void* ws = null
   } else if (dtype == kDtypeBF16) fsw_gemm_kernel<BF16, MODE><<<(unsigned)grid, kThreads, 0, s>>>(g);
   else fsw_gemm_kernel<FP16, MODE><<<(unsigned)grid, kThreads, 0, s>>>(g);
   hipError_t e = hipGetLastError();
-  if (e != hipSuccess || pl.splits == 1) return e;
+  if (e != hipSuccess) return e;
+  if constexpr (!Cfg<MODE>::kForward) {
+    if (g.tail_count > 0) {
+      const dim3 blocks((unsigned)(kTileFloats / 8192), (unsigned)g.tail_count);
+      if (dtype == kDtypeBF16) fsw_tail_reduce_kernel<BF16, MODE><<<blocks, 256, 0, s>>>(g);
+      else fsw_tail_reduce_kernel<FP16, MODE><<<blocks, 256, 0, s>>>(g);
+      return hipGetLastError();
+    }
+  }
+  if (pl.splits == 1) return e;
   const size_t n = (size_t)g.M * g.N;
   const dim3 blocks((unsigned)((n / 4 + 255) / 256), (unsigned)results);
   if (dtype == kDtypeBF16)
