@@ -85,8 +85,23 @@ int fsw_uses_tiled_kernel(int step, int64_t T, int64_t D, int64_t I, int64_t ldx
     case 3: return fsw::fast_path_ok_forward(p) ? 1 : 0;
     case 1: return fsw::fast_path_ok_input_grad(p) ? 1 : 0;
     case 2: return fsw::fast_path_ok_weight_grad(p) ? 1 : 0;
+    default: break;
+  }
+  // the down projection: y, grad_y [T,D] (ldx)   w_down (ldw)   act, grad_act [T,I] (ldo)   grad_w_down (ld_grad)
+  const bool oi = p.w_out_in;
+  fsw::GemmProblem q{ptr, ptr, (void*)ptr, 0, 0, 0, 0, 0, 0, 0};
+  switch (step & 0xff) {
+    case 4: q.M = T; q.N = D; q.K = I; q.lda = ldo; q.ldb = ldw; q.ldc = ldx; q.layout = oi ? 1 : 0; break;
+    case 5: q.M = T; q.N = I; q.K = D; q.lda = ldx; q.ldb = ldw; q.ldc = ldo; q.layout = oi ? 0 : 1; break;
+    case 6:
+      q.layout = 2; q.K = T; q.ldc = ld_grad;
+      if (oi) { q.M = D; q.N = I; q.lda = ldx; q.ldb = ldo; }
+      else { q.M = I; q.N = D; q.lda = ldo; q.ldb = ldx; }
+      break;
     default: return 0;
   }
+  if (!fsw::fast_path_ok_gemm(q)) return 0;
+  return fsw::skinny_gemm_ok(q) ? 2 : 1;
 }
 
 int64_t fsw_workspace_bytes(int step, int64_t T, int64_t D, int64_t I) {
@@ -339,7 +354,9 @@ int fsw_input_grad_noalloc(const void* grad_xw_gate, const void* grad_xw_up, con
   const char* fn = "fsw_input_grad_noalloc";
   if (int e = check_input_grad_args(fn, grad_xw_gate, grad_xw_up, w_gate, w_up, grad_x, T, D, I, ldo, ldw, ld_dx, dtype))
     return e;
-  const int64_t need = fsw::splitk_workspace_bytes(out_in_of(dtype) ? 4 : 1, T, D, I);
+  // only the split reduction of small problems needs its scratch; a large problem whose optional tail split
+  // would not fit the buffer simply runs without it
+  const int64_t need = fsw::splitk_workspace_bytes(out_in_of(dtype) ? 4 : 1, T, D, I, /*with_tail=*/false);
   if (need > (int64_t)FSW_NOALLOC_SCRATCH_BYTES)
     return fail(FSW_ERR_SCRATCH_LIMIT,
                 "%s: T=%lld D=%lld I=%lld needs %lld bytes of split-reduction scratch, the built-in buffer holds %lld; "

@@ -44,8 +44,9 @@ hipError_t launch_forward_fast(int dtype, const Problem& p, hipStream_t s);
 hipError_t launch_input_grad_fast(int dtype, const Problem& p, hipStream_t s, void* ws, long long ws_bytes);
 hipError_t launch_weight_grad_fast(int dtype, const Problem& p, hipStream_t s, void* ws, long long ws_bytes);
 // Bytes of fp32 scratch that let small input-grad (step 1; 4 for [I,D] weights) / weight-grad (step 2; 5)
-// problems split their reduction.
-long long splitk_workspace_bytes(int step, long long T, long long D, long long I);
+// problems split their reduction and, with_tail, large ones share the tiles of a short last round (at most
+// 64 MiB; without that scratch they run exactly as before).
+long long splitk_workspace_bytes(int step, long long T, long long D, long long I, bool with_tail = true);
 
 // Weight-streaming forward for T <= 128 tokens (same eligibility as the tiled forward otherwise).
 bool skinny_forward_ok(const Problem& p);

@@ -10,6 +10,7 @@
 // of the current one, and a slot goes back to the loader as soon as its fragments are in registers.
 #include "fsw_gemm.hpp"
 #include "fsw_internal.hpp"
+#include <atomic>
 
 namespace fsw {
 
@@ -243,11 +244,18 @@ static int block_width(int N, int cus, bool w_kc, int bm) {
   return best;
 }
 
+// Compute units of the current device, looked up once per device (these launches are 75-150 us kernels on the
+// latency-critical decode path).  The plan of a launch depends on it, so a workspace query and the launch it
+// sizes must run with the same device current.
 static int cu_count() {
-  int dev = 0, cus = 0;
-  if (hipGetDevice(&dev) != hipSuccess ||
-      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
-    cus = 256;
+  constexpr int kMaxDevices = 64;
+  static std::atomic<int> cached[kMaxDevices];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+  int cus = cached[dev].load(std::memory_order_relaxed);
+  if (cus > 0) return cus;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+  cached[dev].store(cus, std::memory_order_relaxed);
   return cus;
 }
 

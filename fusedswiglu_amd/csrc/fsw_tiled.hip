@@ -99,20 +99,20 @@ static int steps_of(int mode, long long K) {
 
 // Scratch for a GEMM of the given mode with results `results` x [M, N] and a reduction of K per pass.
 template <int MODE>
-static long long workspace_of(long long M, long long N, long long K) {
+static long long workspace_of(long long M, long long N, long long K, bool with_tail = true) {
   using C = Cfg<MODE>;
   const long long tiles = ((M + C::kTileM - 1) / C::kTileM) * ((N + C::kTileN - 1) / C::kTileN);
   const SplitPlan pl = plan_split_unbounded(tiles, steps_of(MODE, K), M, N, C::kResults);
   if (pl.splits > 1) return (long long)pl.splits * M * N * 4 * C::kResults;
-  return tail_bytes(plan_tail(tiles, steps_of(MODE, K)));
+  return with_tail ? tail_bytes(plan_tail(tiles, steps_of(MODE, K))) : 0;
 }
 
-long long splitk_workspace_bytes(int step, long long T, long long D, long long I) {
+long long splitk_workspace_bytes(int step, long long T, long long D, long long I, bool with_tail) {
   switch (step) {
-    case 1: return workspace_of<kDx>(T, D, I);    // input_grad: result [T, D], reduction over 2*I
-    case 2: return workspace_of<kDw>(D, I, T);    // weight_grad: results 2 x [D, I], reduction over T
-    case 4: return workspace_of<kDxT>(T, D, I);   // the same two for [I, D] weights
-    case 5: return workspace_of<kDwT>(I, D, T);
+    case 1: return workspace_of<kDx>(T, D, I, with_tail);    // input_grad: result [T, D], reduction over 2*I
+    case 2: return workspace_of<kDw>(D, I, T, with_tail);    // weight_grad: results 2 x [D, I], reduction over T
+    case 4: return workspace_of<kDxT>(T, D, I, with_tail);   // the same two for [I, D] weights
+    case 5: return workspace_of<kDwT>(I, D, T, with_tail);
     default: return 0;
   }
 }

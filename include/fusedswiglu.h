@@ -41,15 +41,20 @@
 extern "C" {
 #endif
 
-#define FSW_VERSION 200 /* major*10000 + minor*100 + patch */
+/* major*10000 + minor*100 + patch.
+ * 0.3.0: FSW_WEIGHTS_OUT_IN, the fsw_down_proj_* entry points, fsw_input_grad_noalloc and status 7,
+ *        fsw_uses_tiled_kernel answers 2 for the weight-streaming kernels and knows steps 4 / 5 / 6,
+ *        fsw_workspace_bytes may ask for up to 64 MiB for large gradient GEMMs (tail split).
+ * 0.2.0: fsw_gating_grad_recompute. */
+#define FSW_VERSION 300
 
 enum { FSW_DTYPE_BF16 = 0, FSW_DTYPE_FP16 = 1 };
 /* May be OR-ed into any `dtype` argument (and into the `step` of fsw_workspace_bytes): the weights of the
  * call - w_gate, w_up, w_down and their gradients - are stored "out x in" like torch.nn.Linear.weight, i.e.
  * w_gate, w_up [I, D] and w_down [D, I], instead of the reference's "in x out" ([D, I]; README.md:26-27,
  * fused_swiglu/test_swiglu.py:30-35).  `ldw` / `ld_dw` are then leading dimensions of those arrays.  Nothing is
- * transposed in memory: other tiled-kernel variants read and write the layout in place (the weight-streaming
- * forward for T <= 128 exists for the default layout only). */
+ * transposed in memory: other variants of the tiled kernels and of the weight-streaming kernel (T <= 128) read
+ * and write the layout in place. */
 #define FSW_WEIGHTS_OUT_IN 0x100
 
 enum {
@@ -70,8 +75,12 @@ FSW_API const char* fsw_status_string(int status);
 /* Message of the calling thread's most recent failed call ("" if none). */
 FSW_API const char* fsw_last_error(void);
 /* Which kernel the arguments of the named step would run on: 1 the tiled MFMA kernels, 2 the
- * weight-streaming forward (step 0 with at most 128 tokens), 0 the edge-shape kernel.
- * step: 0 forward, 1 input_grad, 2 weight_grad, 3 gating_grad_recompute.  Pure host logic. */
+ * weight-streaming kernel (at most 128 tokens: the forward, and the down projection and its input gradient
+ * when half their result columns are a multiple of 8 elements for a k-contiguous W_down - [D,I] in the
+ * forward, [I,D] in the input gradient - and of 64 otherwise), 0 the edge-shape kernel.
+ * step: 0 forward, 1 input_grad, 2 weight_grad, 3 gating_grad_recompute, 4 / 5 / 6 down projection forward /
+ * input gradient / weight gradient, each optionally | FSW_WEIGHTS_OUT_IN.  ldx: the [T,D] arrays, ldw: the
+ * weights, ldo: the [T,I] arrays, ld_grad: grad_x or the weight gradient.  Pure host logic. */
 FSW_API int fsw_uses_tiled_kernel(int step, int64_t T, int64_t D, int64_t I, int64_t ldx, int64_t ldw,
                           int64_t ldo, int64_t ld_grad, unsigned pointer_alignment);
 
@@ -114,10 +123,13 @@ FSW_API int fsw_gating_grad_recompute(const void* x, const void* w_gate, const v
  * Optional scratch for the two gradient GEMMs.  When a problem has too few output tiles to fill the
  * chip (small d_model), several workgroups split the reduction of one tile, write fp32 partial
  * tiles to `workspace` (device memory owned by the caller, 16-byte aligned, contents irrelevant) and
- * a second kernel adds them in a fixed order.  fsw_workspace_bytes gives a sufficient size for
+ * a second kernel adds them in a fixed order.  Large problems whose tiles leave a short last round of
+ * workgroups use it the same way for the tiles of that round only (at most 64 MiB).  The few-token down
+ * projection plans its split with the compute-unit count of the current device: query and call with the
+ * same device current.  fsw_workspace_bytes gives a sufficient size for
  * step 1 (input_grad), 2 (weight_grad), 4 / 5 / 6 (down projection forward / input grad / weight grad),
  * each optionally | FSW_WEIGHTS_OUT_IN; with workspace == NULL or a smaller size the call still
- * works, just without the split.  Large problems never touch the workspace.
+ * works, just without the split.
  */
 FSW_API int64_t fsw_workspace_bytes(int step, int64_t T, int64_t D, int64_t I);
 
@@ -136,9 +148,10 @@ FSW_API int fsw_input_grad(const void* grad_xw_gate, const void* grad_xw_up, con
  * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same
  * arguments and results as fsw_input_grad, but the fp32 scratch of the split reduction is a buffer of
  * FSW_NOALLOC_SCRATCH_BYTES built into the library (one copy per GPU, held until the process ends)
- * instead of a caller workspace; the call itself allocates and frees nothing.  Problems whose
- * fsw_workspace_bytes(1, T, D, I) exceeds that size are rejected with FSW_ERR_SCRATCH_LIMIT (large
- * problems need no scratch at all and always pass).  All calls on one GPU share that GPU's buffer:
+ * instead of a caller workspace; the call itself allocates and frees nothing.  Small problems whose
+ * split reduction needs more than that size are rejected with FSW_ERR_SCRATCH_LIMIT (large problems need no
+ * scratch and always pass; the optional tail split of a large problem uses the buffer when it fits and is
+ * skipped when it does not).  All calls on one GPU share that GPU's buffer:
  * calls that overlap in time on one GPU (different streams or threads) race on it.  The first call
  * on a device looks the buffer's address up; make that call outside graph capture.
  */

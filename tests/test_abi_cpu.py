@@ -44,7 +44,7 @@ def test_header_symbols_all_exported(L):
         assert getattr(L, name) is not None
     header = open(os.path.join(ROOT, "include", "fusedswiglu.h")).read()
     m = re.search(r"#define FSW_VERSION (\d+)", header)
-    assert L.fsw_version() == int(m.group(1))
+    assert L.fsw_version() == int(m.group(1)) == 300   # 0.3.0: layouts, down projection, no-allocation entry point
     assert "probe" not in header and "force_edge" not in header
     bench = _declared("fusedswiglu_bench.h")
     assert bench == set(_abi.BENCH_SYMBOLS) == _exported(_abi.BENCH_LIBRARY_PATH)
@@ -152,7 +152,19 @@ def test_kernel_selection_logic(L):
     for step in range(4):
         assert t(step, 8192, 4096, 12288, 4096, 12288, 12288, 4096 if step == 1 else 12288, 16) == 1
         assert t(step, 8192, 4096, 11008, 4096, 11008, 11008, 4096 if step == 1 else 11008, 16) == 1
-    assert t(3, 8192, 4096, 11007, 4096, 11007, 11007, 11007, 16) == 0 and t(4, 8, 8, 8, 8, 8, 8, 8, 16) == 0
+    assert t(3, 8192, 4096, 11007, 4096, 11007, 11007, 11007, 16) == 0 and t(7, 8, 8, 8, 8, 8, 8, 8, 16) == 0
+    # the down projection (steps 4 / 5 / 6; ldx: [T,D] arrays, ldw: W_down, ldo: [T,I] arrays): tiled for many
+    # tokens, weight streaming up to 128 tokens when half the result columns are aligned, never for the weight
+    # gradient; W_down [I,D] by default, [D,I] with the layout flag
+    OI = 0x100
+    for step in (4, 5, 6):
+        assert t(step, 8192, 4096, 12288, 4096, 4096, 12288, 4096, 16) == 1
+        assert t(step | OI, 8192, 4096, 12288, 4096, 12288, 12288, 12288, 16) == 1
+        assert t(step, 8192, 4096, 12281, 4096, 4096, 12281, 4096, 16) == 0
+    assert t(4, 16, 8192, 28672, 8192, 8192, 28672, 8192, 16) == 2 and t(4 | OI, 128, 8192, 28672, 8192, 28672, 28672, 28672, 16) == 2
+    assert t(5, 16, 8192, 28672, 8192, 8192, 28672, 8192, 16) == 2 and t(6, 16, 8192, 28672, 8192, 8192, 28672, 8192, 16) == 1
+    assert t(5, 16, 8192, 72, 8192, 8192, 72, 8192, 16) == 1 and t(5 | OI, 16, 8192, 136, 8192, 136, 136, 136, 16) == 1
+    assert t(4, 129, 8192, 28672, 8192, 8192, 28672, 8192, 16) == 1
     # dimensions that are not multiples of 8, or unaligned pointers, take the edge-shape kernel
     assert t(0, 8192, 4096, 11007, 4096, 11007, 11007, 11007, 16) == 0
     assert t(0, 8192, 4100, 12288, 4100, 12288, 12288, 12288, 16) == 0

@@ -23,7 +23,7 @@ SHAPES = [
     (2, 33, 72, 65),       # I not a multiple of 8 -> edge-shape kernel
     (1, 257, 100, 130),    # nothing aligned
     (4, 512, 256, 768),    # few output tiles, long reductions: split reductions in every gradient GEMM
-    (1, 64, 4096, 1024),   # few tokens: the [I, D] layout has no weight-streaming kernel, the tiled one runs
+    (1, 64, 4096, 1024),   # few tokens: the weight-streaming kernels in either layout, the down projection with a split
 ]
 
 
@@ -122,18 +122,29 @@ def test_down_projection_launchers(oracle, dtype, out_in, shape):
     assert oracle.rel_error(np64(d_w), o_dw.T if out_in else o_dw) < tol
 
 
-FEW_TOKENS_DOWN = [(1, 72, 128), (16, 520, 256), (33, 1096, 384), (64, 4104, 512), (100, 8200, 1024), (128, 2056, 1152)]
+# (T, I, D); the last three have I a multiple of 128, so that the input gradient streams W_down as well (half of
+# its I result columns must be a multiple of 64, or of 8 for [I, D] storage), with and without a split reduction
+FEW_TOKENS_DOWN = [(1, 72, 128), (16, 520, 256), (33, 1096, 384), (64, 4104, 512), (100, 8200, 1024), (128, 2056, 1152),
+                   (16, 1024, 4096), (64, 28672, 1024), (128, 256, 8192)]
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 @pytest.mark.parametrize("out_in", [False, True], ids=["w_down_IxD", "w_down_DxI"])
 @pytest.mark.parametrize("tid", FEW_TOKENS_DOWN, ids=lambda s: "x".join(map(str, s)))
 def test_few_token_down_projection(oracle, dtype, out_in, tid):
-    """Up to 128 tokens the down projection (and its input gradient) streams the weights on the kernel of the
-    few-token forward, as a plain GEMM over the two column halves of W_down with the reduction split into the
-    caller's scratch: against the oracle with scratch (the launcher asks the library for it), and through the
-    raw ABI without scratch (no split), which must agree to within the rounding of one more fp32 summation order."""
+    """Up to 128 tokens the down projection streams the weights on the kernel of the few-token forward, as a plain
+    GEMM over the two column halves of W_down with the reduction split into the caller's scratch; so does its
+    input gradient when half of I is aligned (selection code 2, else the tiled kernel, code 1): against the oracle
+    with scratch (the launcher asks the library for it), and through the raw ABI without scratch (no split), which
+    must agree to within the rounding of one more fp32 summation order."""
     T, I, D = tid
+    flag = _abi.WEIGHTS_OUT_IN if out_in else 0
+    uses = _abi.lib().fsw_uses_tiled_kernel
+    ldw = I if out_in else D
+    assert uses(4 | flag, T, D, I, D, ldw, I, ldw, 16) == 2      # D / 2 is a multiple of 64 in every case
+    half_ok = (I // 2) % (64 if out_in else 8) == 0 and I % 2 == 0
+    assert uses(5 | flag, T, D, I, D, ldw, I, ldw, 16) == (2 if half_ok else 1)
+    assert uses(6 | flag, T, D, I, D, ldw, I, ldw, 16) == 1
     rng = np.random.default_rng(T + I)
     rnd = oracle.rounder(NAME[dtype])
     act = rnd(rng.standard_normal((T, I)))
