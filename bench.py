@@ -27,7 +27,7 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # itself).  The summary is stamped with a hash of the kernel sources it was taken with; when the sources
 # have changed since, `traffic` is reported as null instead of a stale figure.
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "gemm_kernels_c2_bf16.md")
-KERNEL_SOURCES = ("fsw_common.hpp", "fsw_gemm.hpp", "fsw_tiled.hip")
+KERNEL_SOURCES = ("fsw_common.hpp", "fsw_gemm.hpp", "fsw_gemm4.hpp", "fsw_tiled.hip")
 
 
 def kernel_source_hash():
@@ -67,8 +67,8 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the skinny-M and per-kernel extras")
     ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run three plain 1 GiB device copies (known HBM traffic) so that profiler "
-                         "byte counters collected over this run can be scaled")
+                    help="also run launches of known HBM traffic (1 GiB plain copies, streaming reads and "
+                         "direct-to-LDS reads) so that profiler byte counters collected over this run can be scaled")
     return ap.parse_args()
 
 
@@ -277,15 +277,25 @@ def main():
         del window
         big = torch.empty(1 << 31, device=dev, dtype=torch.uint8).fill_(1)
         ms = gpu_time_ms(lambda: _abi.check(_abi.bench_lib().fsw_probe_stream_read(p(big), big.numel(), p(sink), stream)), iters=5, warmup=2)
-        ceil["hbm_stream_read_gbs"] = round(big.numel() / ms / 1e6, 1)
+        # the rate of a plain streaming-read kernel, for orientation: not a bound (the weight-streaming kernels
+        # and the elementwise kernel may exceed it)
+        ceil["hbm_read_probe_gbs"] = round(big.numel() / ms / 1e6, 1)
         del big
         result["measured_ceilings"] = ceil
 
     if args.calibrate_copy:
+        # launches of known HBM traffic (1 GiB each, far beyond the caches), three of each: a plain copy, a
+        # streaming read, and the kernels' own request pattern (direct global->LDS loads of whole lines, without
+        # and with the non-temporal hint)
         src = torch.empty(1 << 30, device=dev, dtype=torch.uint8).fill_(1)
         dst = torch.empty_like(src)
+        sink = torch.zeros(4, device=dev, dtype=torch.float32)
+        B = _abi.bench_lib()
         for _ in range(3):
             dst.copy_(src)
+            _abi.check(B.fsw_probe_stream_read(p(dst), dst.numel(), p(sink), stream))
+            _abi.check(B.fsw_probe_dma_read(p(src), src.numel(), 0, stream))
+            _abi.check(B.fsw_probe_dma_read(p(dst), dst.numel(), 1, stream))
         torch.cuda.synchronize()
         del src, dst
 

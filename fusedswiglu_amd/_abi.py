@@ -46,7 +46,7 @@ EXPORTED_SYMBOLS = (
     "fsw_down_proj_weight_grad",
 )
 #: every symbol include/fusedswiglu_bench.h declares (libfusedswiglu_bench.so)
-BENCH_SYMBOLS = ("fsw_probe_mfma", "fsw_probe_stream_read", "fsw_probe_mfma_mix")
+BENCH_SYMBOLS = ("fsw_probe_mfma", "fsw_probe_stream_read", "fsw_probe_mfma_mix", "fsw_probe_dma_read")
 
 
 class FusedSwiGLUError(RuntimeError):
@@ -142,6 +142,7 @@ def bench_lib() -> ctypes.CDLL:
             L.fsw_probe_mfma.argtypes = [ci, ci, ci, vp, vp, ctypes.POINTER(ctypes.c_double)]
             L.fsw_probe_stream_read.restype = ci
             L.fsw_probe_stream_read.argtypes = [vp, i64, vp, vp]
+            L.fsw_probe_dma_read.argtypes = [vp, i64, ci, vp]
             L.fsw_probe_mfma_mix.restype = ci
             L.fsw_probe_mfma_mix.argtypes = [ci, ci, ci, vp, i64, vp, vp, ctypes.POINTER(ctypes.c_double)]
             _bench_lib = L

@@ -107,13 +107,37 @@ __global__ __launch_bounds__(256) void probe_read_kernel(const u32x4* __restrict
   const size_t stride = (size_t)gridDim.x * blockDim.x;
   unsigned s = 0;
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  for (; i + 3 * stride < n16; i += 4 * stride) {
-    const u32x4 a = __builtin_nontemporal_load(p + i), b = __builtin_nontemporal_load(p + i + stride),
-                c = __builtin_nontemporal_load(p + i + 2 * stride), d = __builtin_nontemporal_load(p + i + 3 * stride);
-    s += a[0] ^ a[1] ^ a[2] ^ a[3] ^ b[0] ^ b[1] ^ b[2] ^ b[3] ^ c[0] ^ c[1] ^ c[2] ^ c[3] ^ d[0] ^ d[1] ^ d[2] ^ d[3];
+  for (; i + 7 * stride < n16; i += 8 * stride) {
+    u32x4 v[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) v[k] = __builtin_nontemporal_load(p + i + k * stride);
+#pragma unroll
+    for (int k = 0; k < 8; k++) s += v[k][0] ^ v[k][1] ^ v[k][2] ^ v[k][3];
   }
   for (; i < n16; i += stride) { const u32x4 a = p[i]; s += a[0] ^ a[1] ^ a[2] ^ a[3]; }
   if (s == 0x12345678u) sink[0] = s;
+}
+
+// The tiled and the weight-streaming kernels' way of reading: direct global->LDS loads of 1 KiB per wave (eight
+// rows of one 128-byte line), every byte of the buffer exactly once, optionally with the non-temporal hint.  The
+// descriptor carries the exact size, so no lane can read outside the buffer.  Known traffic for calibrating the
+// profiler's byte counters against this request pattern.
+template <bool NT>
+__global__ __launch_bounds__(256) void probe_dma_read_kernel(const char* buf, unsigned bytes) {
+  __shared__ __attribute__((aligned(1024))) char smem[32 * 1024];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const i32x4 rs = make_rsrc(buf, bytes);
+  const unsigned lds = (unsigned)(uintptr_t)(FSW_LDS char*)smem + wave * 8192;
+  const unsigned chunks = bytes >> 10, waves = gridDim.x * 4;
+  int k = 0;
+  for (unsigned c = blockIdx.x * 4 + wave; c < chunks; c += waves, k++) {
+    const unsigned off = c * 1024u + lane * 16u;
+    if (NT) load16_to_lds_stream(rs, off, lds + (k & 7) * 1024);
+    else load16_to_lds(rs, off, lds + (k & 7) * 1024);
+    if ((k & 7) == 7) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
 }  // namespace fsw
@@ -151,6 +175,13 @@ int fsw_probe_mfma_mix(int mix, int iters, int workgroups, const void* buf, int6
 int fsw_probe_stream_read(const void* buf, int64_t bytes, void* sink4, void* stream) {
   if (!buf || !sink4 || bytes < 16 || ((uintptr_t)buf & 15)) return FSW_ERR_BAD_SHAPE;
   fsw::probe_read_kernel<<<4096, 256, 0, (hipStream_t)stream>>>((const fsw::u32x4*)buf, (size_t)bytes / 16, (unsigned*)sink4);
+  return hipGetLastError() == hipSuccess ? FSW_OK : FSW_ERR_LAUNCH;
+}
+
+int fsw_probe_dma_read(const void* buf, int64_t bytes, int non_temporal, void* stream) {
+  if (!buf || bytes < 1024 || bytes > 0x7fffffffLL || (bytes & 1023) || ((uintptr_t)buf & 15)) return FSW_ERR_BAD_SHAPE;
+  if (non_temporal) fsw::probe_dma_read_kernel<true><<<2048, 256, 0, (hipStream_t)stream>>>((const char*)buf, (unsigned)bytes);
+  else fsw::probe_dma_read_kernel<false><<<2048, 256, 0, (hipStream_t)stream>>>((const char*)buf, (unsigned)bytes);
   return hipGetLastError() == hipSuccess ? FSW_OK : FSW_ERR_LAUNCH;
 }
 
