@@ -18,6 +18,9 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
 #define FSW_LDS __attribute__((address_space(3)))
 #define FSW_DEV __device__ __forceinline__
@@ -39,6 +42,12 @@ struct BF16 {
   static FSW_DEV unsigned short from_float(float f) {
     return __builtin_bit_cast(unsigned short, (__bf16)f);
   }
+  // two values in one v_cvt_pk_bf16_f32 (same rounding): `lo` in bits 0..15.  Through the compiler and not as
+  // inline assembly: it knows the wait state this instruction needs before an LDS or memory instruction reads
+  // its result (without it, some lanes store the unconverted input).
+  static FSW_DEV unsigned pack2(float lo, float hi) {
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2{lo, hi}, bf16x2));
+  }
 };
 struct FP16 {
   using vec8 = f16x8;
@@ -55,6 +64,10 @@ struct FP16 {
   }
   static FSW_DEV unsigned short from_float(float f) {
     return __builtin_bit_cast(unsigned short, (_Float16)f);
+  }
+  // two values in one v_cvt_pk_f16_f32 (same rounding): `lo` in bits 0..15
+  static FSW_DEV unsigned pack2(float lo, float hi) {
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2{lo, hi}, f16x2));
   }
 };
 

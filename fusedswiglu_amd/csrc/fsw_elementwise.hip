@@ -32,11 +32,11 @@ __global__ __launch_bounds__(256) void elementwise_backward_kernel(
     u32x4 ru, rg;
 #pragma unroll
     for (int w = 0; w < 4; w++) {
-      unsigned short u0, g0, u1, g1;
-      gate_grad<E>(a[w] & 0xffff, b[w] & 0xffff, c[w] & 0xffff, u0, g0);
-      gate_grad<E>(a[w] >> 16, b[w] >> 16, c[w] >> 16, u1, g1);
-      ru[w] = u0 | ((unsigned)u1 << 16);
-      rg[w] = g0 | ((unsigned)g1 << 16);
+      float u0, g0, u1, g1;
+      gating_grad(E::to_float(a[w] & 0xffff), E::to_float(b[w] & 0xffff), E::to_float(c[w] & 0xffff), u0, g0);
+      gating_grad(E::to_float(a[w] >> 16), E::to_float(b[w] >> 16), E::to_float(c[w] >> 16), u1, g1);
+      ru[w] = E::pack2(u0, u1);
+      rg[w] = E::pack2(g0, g1);
     }
     __builtin_nontemporal_store(ru, (u32x4*)dU + v);
     __builtin_nontemporal_store(rg, (u32x4*)dG + v);

@@ -27,6 +27,7 @@
 // the pair, and the fragment reads of a step are always one step ahead of the MFMAs that consume them.
 #pragma once
 #include <type_traits>
+#include <utility>
 
 #include "fsw_common.hpp"
 
@@ -200,6 +201,185 @@ FSW_DEV void mc_setup(McLoader& L, const void* p_panel0, const void* p_panel1, c
 }
 
 // STREAM_B: the B operand is read once by the whole launch (a single row of tiles): load it non-temporally
+template <int... I, typename F>
+FSW_DEV void static_for_impl(std::integer_sequence<int, I...>, F&& f) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+FSW_DEV void static_for(F&& f) {
+  static_for_impl(std::make_integer_sequence<int, N>{}, f);
+}
+
+// ---- the epilogue of both forms of the tiled kernel: rounding, silu(g) * u or the gating gradients, and whole
+// 128-byte lines to memory.
+//
+// A wave holds 32*NQ rows x 128 columns of accumulators: acc[nb][mb][r] of lane l is the wave's row
+// mb*16 + (l & 15) and, within the wave's half h = nb >> 2, column (nb & 3)*16 + 4*(l >> 4) + r of 64 consecutive
+// result columns (128 bytes).  Half h goes to result res_half[h] (0: c0, 1: c1) at columns col_half[h]..; in the
+// forwards the two halves are gate and up of the same 64 columns col_half[0].
+//
+// The work is a sequence of "parts" (32 rows x 64 columns of one result each) in a software pipeline: while the
+// values of part k are computed and written into LDS patch k & 1 (32 rows x 128 bytes; 16-byte chunk c of row r
+// sits at position c ^ ((r >> 1) & 7), so neither the 8-byte accumulator writes nor the 16-byte row reads
+// conflict), the lines of part k-1 are on their way from the other patch to memory.  Everything is branch free -
+// edges are masked through the offsets of buffer stores and loads, which the descriptors' range check drops - so
+// the whole epilogue is one basic block that the compiler schedules across parts.  The results are written once
+// and read by a later kernel at the earliest: non-temporal stores keep them out of the way of the operands.
+//
+// ACC_ASM: the accumulators live in the accumulation registers behind inline-asm MFMAs (four-wave form); they are
+// then moved out by explicit instructions at their turn and not earlier (left to the compiler, they are moved out
+// wholesale after the main loop and spill).
+template <typename E, int MODE, int NQ, bool ACC_ASM>
+FSW_DEV void store_tile(const GemmParams& p, f32x4 (&acc)[8][2 * NQ], FSW_LDS char* patch, int lane, int row_base,
+                        int col_half0, int col_half1, int res_half0, int res_half1) {
+  using C = Cfg<MODE>;
+  constexpr int kPatchPitch = 128, kPatchBytes = 32 * kPatchPitch;
+  const int wr_row = (lane & 15) * kPatchPitch, wr_swz = (lane >> 1) & 7, wr_grp = lane >> 4;
+  // 8 bytes of column group wr_grp of 16-column block c:  chunk 2c + (wr_grp >> 1), half wr_grp & 1
+  auto wr_off = [&](int mbl, int c) {
+    return mbl * 16 * kPatchPitch + wr_row + (((2 * c + (wr_grp >> 1)) ^ wr_swz) << 4) + (wr_grp & 1) * 8;
+  };
+  // row 8i + (lane >> 3), chunk lane & 7
+  auto rd_off = [&](int i) {
+    const int row = 8 * i + (lane >> 3);
+    return row * kPatchPitch + (((lane & 7) ^ ((row >> 1) & 7)) << 4);
+  };
+  const int rows_left = p.M - row_base;             // rows of this wave that exist (may be <= 0 or >= 32*NQ)
+  const unsigned ldc_bytes = (unsigned)p.ldc * 2u;  // the host keeps 128 rows of a result below 2^31 bytes
+  // a result seen from the wave's first row and column `col_base`
+  auto result_rsrc = [&](const void* base, int col_base) {
+    return __builtin_amdgcn_make_buffer_rsrc((char*)base + ((size_t)row_base * p.ldc + col_base) * 2, 0, 0x7fffffff,
+                                             kRsrcWord3);
+  };
+  // line store i of a part: lane l holds chunk l & 7 of row 8*i + (l >> 3) of the part's 32 rows
+  const unsigned st_lane = (unsigned)(lane >> 3) * ldc_bytes + (unsigned)(lane & 7) * 16u;
+  u32x4 in_flight[4];
+  auto read_part = [&](int k) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) in_flight[i] = *(const FSW_LDS u32x4*)(patch + (k & 1) * kPatchBytes + rd_off(i));
+  };
+  // st_cols: st_lane, or the out-of-range offset in lanes whose columns do not exist
+  auto store_part = [&](__amdgpu_buffer_rsrc_t rs, unsigned st_cols, int q) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int r0 = q * 32 + 8 * i;
+      // The row offset goes through the vector offset, not the scalar one: behind a 16-byte store with a scalar
+      // offset REGISTER the compiler leaves out the wait state before the next instruction that overwrites the
+      // store's data registers, and on this hardware the store then picks up the new value in some lanes.
+      const unsigned off = ((lane >> 3) < rows_left - r0 ? st_cols : kOobOffset) + (unsigned)r0 * ldc_bytes;
+      __builtin_amdgcn_raw_buffer_store_b128(in_flight[i], rs, off, 0, 2 /* nt */);
+    }
+  };
+  auto write_part = [&](int k, int mbl, int c, float a, float b, float cc, float d) {
+    u32x2 v;
+    v.x = E::pack2(a, b);
+    v.y = E::pack2(cc, d);
+    *(FSW_LDS u32x2*)(patch + (k & 1) * kPatchBytes + wr_off(mbl, c)) = v;
+  };
+  auto acc_read = [&](float a) {
+    if constexpr (ACC_ASM) {
+      float v;
+      asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
+      return v;
+    } else {
+      return a;
+    }
+  };
+  auto acc_read4 = [&](const f32x4& a) { return f32x4{acc_read(a.x), acc_read(a.y), acc_read(a.z), acc_read(a.w)}; };
+  if constexpr (C::kForward) {
+    const int colw = col_half0;
+    const unsigned st_cols = colw + (lane & 7) * 8 < p.N ? st_lane : kOobOffset;
+    // first: 0 = out, g, u (or out alone when the caller passes no buffers for g and u); 1 = dG, dU from dout
+    // (gating-gradient mode, d0 given).  Compile-time parameters, so that the parts carry no branch on them.
+    auto forward_tile = [&](auto first_tag, auto count_tag) {
+      constexpr int first = decltype(first_tag)::value, count = decltype(count_tag)::value;
+      constexpr bool gating = first == 1;
+      __amdgpu_buffer_rsrc_t rs[3] = {result_rsrc(p.c0, colw), result_rsrc(count > 1 ? p.c1 : p.c0, colw),
+                                      result_rsrc(count > 1 ? p.c2 : p.c0, colw)};
+      __amdgpu_buffer_rsrc_t rs_d = result_rsrc(gating ? p.d0 : p.c0, colw);
+      // dout in the accumulator layout: 4 consecutive columns of row (l & 15) per lane and 16x16 block
+      const unsigned ld_lane = (unsigned)(lane & 15) * ldc_bytes + (unsigned)(lane >> 4) * 8u;
+      unsigned ld_cols[4];
+#pragma unroll
+      for (int c = 0; c < 4; c++) ld_cols[c] = colw + c * 16 + 4 * (lane >> 4) < p.N ? ld_lane + c * 32u : kOobOffset;
+      u32x2 dv[2][4];
+      f32x4 gq[2][4], uq[2][4];  // the gate and up values of the 32 rows in hand
+      static_for<NQ * count>([&](auto kc) {
+        constexpr int k = decltype(kc)::value, q = k / count, which = first + k % count;
+        if constexpr (k % count == 0) {
+#pragma unroll
+          for (int mbl = 0; mbl < 2; mbl++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+              gq[mbl][c] = acc_read4(acc[c][2 * q + mbl]);
+              uq[mbl][c] = acc_read4(acc[4 + c][2 * q + mbl]);
+            }
+          if constexpr (gating) {
+#pragma unroll
+            for (int mbl = 0; mbl < 2; mbl++)
+#pragma unroll
+              for (int c = 0; c < 4; c++) {
+                const int r0 = (2 * q + mbl) * 16;
+                const unsigned off = (lane & 15) < rows_left - r0 ? ld_cols[c] : kOobOffset;
+                dv[mbl][c] = __builtin_amdgcn_raw_buffer_load_b64(rs_d, off, (unsigned)r0 * ldc_bytes, 0);
+              }
+          }
+        }
+        if constexpr (k > 0) read_part(k - 1);
+#pragma unroll
+        for (int mbl = 0; mbl < 2; mbl++)
+#pragma unroll
+          for (int c = 0; c < 4; c++) {
+            const f32x4 g = gq[mbl][c], u = uq[mbl][c];
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              if constexpr (gating) {
+                const unsigned w = e < 2 ? dv[mbl][c].x : dv[mbl][c].y;
+                float dU, dG;
+                gating_grad(E::to_float((unsigned short)((e & 1) ? (w >> 16) : (w & 0xffffu))), g[e], u[e], dU, dG);
+                v[e] = which == 1 ? dG : dU;
+              } else {
+                v[e] = which == 0 ? silu_mul(g[e], u[e]) : (which == 1 ? g[e] : u[e]);
+              }
+            }
+            write_part(k, mbl, c, v[0], v[1], v[2], v[3]);
+          }
+        if constexpr (k > 0) store_part(rs[first + (k - 1) % count], st_cols, (k - 1) / count);
+      });
+      read_part(NQ * count - 1);
+      store_part(rs[first + count - 1], st_cols, NQ - 1);
+    };
+    if (p.d0 != nullptr) forward_tile(std::integral_constant<int, 1>{}, std::integral_constant<int, 2>{});
+    else if (p.c1 != nullptr) forward_tile(std::integral_constant<int, 0>{}, std::integral_constant<int, 3>{});
+    else forward_tile(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{});
+  } else {
+    __amdgpu_buffer_rsrc_t rs[2] = {result_rsrc(res_half0 == 0 ? p.c0 : p.c1, col_half0),
+                                    result_rsrc(res_half1 == 0 ? p.c0 : p.c1, col_half1)};
+    const unsigned st_cols[2] = {col_half0 + (lane & 7) * 8 < p.N ? st_lane : kOobOffset,
+                                 col_half1 + (lane & 7) * 8 < p.N ? st_lane : kOobOffset};
+    static_for<2 * NQ>([&](auto kc) {
+      constexpr int k = decltype(kc)::value, q = k >> 1, h = k & 1;
+      if constexpr (ACC_ASM) {
+        // (one result per half: pinning the registers costs a copy, which two or three tiles per launch do not feel)
+#pragma unroll
+        for (int c = 0; c < 4; c++) asm volatile("" : "+a"(acc[4 * h + c][2 * q]), "+a"(acc[4 * h + c][2 * q + 1]));
+      }
+      if constexpr (k > 0) read_part(k - 1);
+#pragma unroll
+      for (int mbl = 0; mbl < 2; mbl++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+          const f32x4 t = acc[4 * h + c][2 * q + mbl];
+          write_part(k, mbl, c, t[0], t[1], t[2], t[3]);
+        }
+      if constexpr (k > 0) store_part(rs[(k - 1) & 1], st_cols[(k - 1) & 1], (k - 1) >> 1);
+    });
+    read_part(2 * NQ - 1);
+    store_part(rs[1], st_cols[1], NQ - 1);
+  }
+}
+
 template <typename E, int MODE, bool STREAM_B = false>
 __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
   using C = Cfg<MODE>;
@@ -409,104 +589,8 @@ __global__ __launch_bounds__(kThreads) void fsw_gemm_kernel(GemmParams p) {
     }
     return;
   }
-  // patch: 32 rows x 128 bytes per wave; 16-byte chunk c of row r sits at position c ^ ((r >> 1) & 7), which
-  // keeps both the 8-byte accumulator writes (16 rows x 4 column groups per instruction) and the 16-byte
-  // row reads (2 rows x 128 bytes per 16 lanes) free of bank conflicts
-  constexpr int kPatchPitch = 128;
-  FSW_LDS char* patch = (FSW_LDS char*)smem + wave * (32 * kPatchPitch);
-  const int wr_row = (lane & 15) * kPatchPitch, wr_swz = (lane >> 1) & 7, wr_grp = lane >> 4;
-  // 8 bytes of column group wr_grp of 16-column block c:  chunk 2c + (wr_grp >> 1), half wr_grp & 1
-  auto wr_off = [&](int mbl, int c) {
-    return mbl * 16 * kPatchPitch + wr_row + (((2 * c + (wr_grp >> 1)) ^ wr_swz) << 4) + (wr_grp & 1) * 8;
-  };
-  // row 8i + (lane >> 3), chunk lane & 7
-  auto rd_off = [&](int i) {
-    const int row = 8 * i + (lane >> 3);
-    return row * kPatchPitch + (((lane & 7) ^ ((row >> 1) & 7)) << 4);
-  };
-  auto flush_patch = [&](unsigned short* dst, int col_base, int q) {
-    // rows q*32 + 8i + (lane >> 3), columns col_base + (lane & 7)*8 .. +8
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const u32x4 v = *(const FSW_LDS u32x4*)(patch + rd_off(i));
-      const int m = row_base + q * 32 + 8 * i + (lane >> 3);
-      const int n = col_base + (lane & 7) * 8;
-      // written once, read by a later kernel at the earliest: keep the lines out of the way of the operands
-      if (m < p.M && n < p.N) __builtin_nontemporal_store(v, (u32x4*)(dst + (size_t)m * p.ldc + n));
-    }
-  };
-  auto pack4 = [&](float a, float b, float c, float d) {
-    u32x2 v;
-    v.x = E::from_float(a) | ((unsigned)E::from_float(b) << 16);
-    v.y = E::from_float(c) | ((unsigned)E::from_float(d) << 16);
-    return v;
-  };
-  if constexpr (C::kForward) {
-    // out = silu(g) * u, then g and u themselves (skipped when the caller passes no buffers for them); in
-    // gating-gradient mode (d0 given) dG and dU take the places of g and u and out is not written.  The mode is
-    // a compile-time parameter of the body so that the inner loops carry no branch on it.
-    auto forward_tile = [&](auto gating_tag) {
-      constexpr bool gating = decltype(gating_tag)::value;
-#pragma unroll
-      for (int q = 0; q < 2; q++) {  // 32 rows of the wave's 64 at a time
-        // gating-gradient mode: this lane's upstream gradients, 4 consecutive columns per 16x16 block
-        u32x2 dv[2][4];
-        if constexpr (gating) {
-#pragma unroll
-          for (int mbl = 0; mbl < 2; mbl++)
-#pragma unroll
-            for (int c = 0; c < 4; c++) {
-              const int m = row_base + (2 * q + mbl) * 16 + (lane & 15);
-              const int n = n0 + wn * 64 + c * 16 + 4 * (lane >> 4);
-              dv[mbl][c] = (m < p.M && n < p.N) ? *(const u32x2*)((const unsigned short*)p.d0 + (size_t)m * p.ldc + n)
-                                                : u32x2{0u, 0u};
-            }
-        }
-#pragma unroll
-        for (int which = gating ? 1 : 0; which < 3; which++) {
-          if (which > 0 && p.c1 == nullptr) break;
-#pragma unroll
-          for (int mbl = 0; mbl < 2; mbl++)
-#pragma unroll
-            for (int c = 0; c < 4; c++) {
-              const f32x4 g = acc[c][2 * q + mbl], u = acc[4 + c][2 * q + mbl];
-              float v[4];
-#pragma unroll
-              for (int e = 0; e < 4; e++) {
-                if constexpr (gating) {
-                  const unsigned w = e < 2 ? dv[mbl][c].x : dv[mbl][c].y;
-                  float dU, dG;
-                  gating_grad(E::to_float((unsigned short)((e & 1) ? (w >> 16) : (w & 0xffffu))), g[e], u[e], dU, dG);
-                  v[e] = which == 1 ? dG : dU;
-                } else {
-                  v[e] = which == 0 ? silu_mul(g[e], u[e]) : (which == 1 ? g[e] : u[e]);
-                }
-              }
-              *(FSW_LDS u32x2*)(patch + wr_off(mbl, c)) = pack4(v[0], v[1], v[2], v[3]);
-            }
-          unsigned short* dst = (unsigned short*)(which == 0 ? p.c0 : (which == 1 ? p.c1 : p.c2));
-          flush_patch(dst, n0 + wn * 64, q);
-        }
-      }
-    };
-    if (p.d0 != nullptr) forward_tile(std::true_type{});
-    else forward_tile(std::false_type{});
-  } else {
-#pragma unroll
-    for (int q = 0; q < 2; q++) {  // 32 rows of the wave's 64 at a time
-#pragma unroll
-      for (int h = 0; h < 2; h++) {  // the wave's two groups of 64 columns
-#pragma unroll
-        for (int mbl = 0; mbl < 2; mbl++)
-#pragma unroll
-          for (int c = 0; c < 4; c++) {
-            const f32x4 t = acc[4 * h + c][2 * q + mbl];
-            *(FSW_LDS u32x2*)(patch + wr_off(mbl, c)) = pack4(t[0], t[1], t[2], t[3]);
-          }
-        flush_patch((unsigned short*)(result_of_half(h) == 0 ? p.c0 : p.c1), col_of_half(h), q);
-      }
-    }
-  }
+  store_tile<E, MODE, 2, false>(p, acc, (FSW_LDS char*)smem + wave * (2 * 32 * 128), lane, row_base, col_of_half(0),
+                                col_of_half(1), result_of_half(0), result_of_half(1));
 }
 
 // out_r[i] = round(sum over s of ws[r][s][i]), i < n, fixed order: deterministic.  n is a multiple of 4.
@@ -526,8 +610,8 @@ __global__ __launch_bounds__(256) void fsw_splitk_reduce_kernel(const float* __r
   }
   const size_t m = i4 / (size_t)N, c = i4 - m * (size_t)N;
   u32x2 v;
-  v.x = E::from_float(a.x) | ((unsigned)E::from_float(a.y) << 16);
-  v.y = E::from_float(a.z) | ((unsigned)E::from_float(a.w) << 16);
+  v.x = E::pack2(a.x, a.y);
+  v.y = E::pack2(a.z, a.w);
   *(u32x2*)(out + m * (size_t)ldc + c) = v;
 }
 

@@ -34,15 +34,6 @@ constexpr int gap_index(int g, int start, int stride, int count) {
   return (g >= start && (g - start) % stride == 0 && (g - start) / stride < count) ? (g - start) / stride : -1;
 }
 
-template <int... I, typename F>
-FSW_DEV void static_for_impl(std::integer_sequence<int, I...>, F&& f) {
-  (f(std::integral_constant<int, I>{}), ...);
-}
-template <int N, typename F>
-FSW_DEV void static_for(F&& f) {
-  static_for_impl(std::make_integer_sequence<int, N>{}, f);
-}
-
 // c += a b with the accumulator pinned to the accumulation registers and the operands to ordinary vector
 // registers.  Left to itself the register allocator mixes the two files for a 128 x 128 wave tile and shuffles
 // accumulators back and forth around every MFMA.
@@ -464,94 +455,8 @@ __global__ __launch_bounds__(kThreads4) void fsw_gemm4_kernel(GemmParams p) {
     }
     return;
   }
-  // patch: 32 rows x 128 bytes per wave; 16-byte chunk c of row r sits at position c ^ ((r >> 1) & 7)
-  constexpr int kPatchPitch = 128;
-  FSW_LDS char* patch = (FSW_LDS char*)smem + wave * (32 * kPatchPitch);
-  const int wr_row = (lane & 15) * kPatchPitch, wr_swz = (lane >> 1) & 7, wr_grp = lane >> 4;
-  auto wr_off = [&](int mbl, int c) {
-    return mbl * 16 * kPatchPitch + wr_row + (((2 * c + (wr_grp >> 1)) ^ wr_swz) << 4) + (wr_grp & 1) * 8;
-  };
-  auto rd_off = [&](int i) {
-    const int row = 8 * i + (lane >> 3);
-    return row * kPatchPitch + (((lane & 7) ^ ((row >> 1) & 7)) << 4);
-  };
-  auto flush_patch = [&](unsigned short* dst, int col_base, int q) {
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const u32x4 v = *(const FSW_LDS u32x4*)(patch + rd_off(i));
-      const int m = row_base + q * 32 + 8 * i + (lane >> 3);
-      const int n = col_base + (lane & 7) * 8;
-      if (m < p.M && n < p.N) __builtin_nontemporal_store(v, (u32x4*)(dst + (size_t)m * p.ldc + n));
-    }
-  };
-  auto pack4 = [&](float a, float b, float c, float d) {
-    u32x2 v;
-    v.x = E::from_float(a) | ((unsigned)E::from_float(b) << 16);
-    v.y = E::from_float(c) | ((unsigned)E::from_float(d) << 16);
-    return v;
-  };
-  if constexpr (C::kForward) {
-    auto forward_tile = [&](auto gating_tag) {
-      constexpr bool gating = decltype(gating_tag)::value;
-#pragma unroll
-      for (int q = 0; q < 4; q++) {  // 32 rows of the wave's 128 at a time
-        u32x2 dv[2][4];
-        if constexpr (gating) {
-#pragma unroll
-          for (int mbl = 0; mbl < 2; mbl++)
-#pragma unroll
-            for (int c = 0; c < 4; c++) {
-              const int m = row_base + (2 * q + mbl) * 16 + (lane & 15);
-              const int n = n0 + wn * 64 + c * 16 + 4 * (lane >> 4);
-              dv[mbl][c] = (m < p.M && n < p.N) ? *(const u32x2*)((const unsigned short*)p.d0 + (size_t)m * p.ldc + n)
-                                                : u32x2{0u, 0u};
-            }
-        }
-#pragma unroll
-        for (int which = gating ? 1 : 0; which < 3; which++) {
-          if (which > 0 && p.c1 == nullptr) break;
-#pragma unroll
-          for (int mbl = 0; mbl < 2; mbl++)
-#pragma unroll
-            for (int c = 0; c < 4; c++) {
-              const f32x4 g = acc[c][2 * q + mbl], u = acc[4 + c][2 * q + mbl];
-              float v[4];
-#pragma unroll
-              for (int e = 0; e < 4; e++) {
-                if constexpr (gating) {
-                  const unsigned w = e < 2 ? dv[mbl][c].x : dv[mbl][c].y;
-                  float dU, dG;
-                  gating_grad(E::to_float((unsigned short)((e & 1) ? (w >> 16) : (w & 0xffffu))), g[e], u[e], dU, dG);
-                  v[e] = which == 1 ? dG : dU;
-                } else {
-                  v[e] = which == 0 ? silu_mul(g[e], u[e]) : (which == 1 ? g[e] : u[e]);
-                }
-              }
-              *(FSW_LDS u32x2*)(patch + wr_off(mbl, c)) = pack4(v[0], v[1], v[2], v[3]);
-            }
-          unsigned short* dst = (unsigned short*)(which == 0 ? p.c0 : (which == 1 ? p.c1 : p.c2));
-          flush_patch(dst, n0 + wn * 64, q);
-        }
-      }
-    };
-    if (p.d0 != nullptr) forward_tile(std::true_type{});
-    else forward_tile(std::false_type{});
-  } else {
-#pragma unroll
-    for (int q = 0; q < 4; q++) {
-#pragma unroll
-      for (int h = 0; h < 2; h++) {
-#pragma unroll
-        for (int mbl = 0; mbl < 2; mbl++)
-#pragma unroll
-          for (int c = 0; c < 4; c++) {
-            const f32x4 t = acc[4 * h + c][2 * q + mbl];
-            *(FSW_LDS u32x2*)(patch + wr_off(mbl, c)) = pack4(t[0], t[1], t[2], t[3]);
-          }
-        flush_patch((unsigned short*)(result_of_half(h) == 0 ? p.c0 : p.c1), col_of_half(h), q);
-      }
-    }
-  }
+  store_tile<E, MODE, 4, true>(p, acc, (FSW_LDS char*)smem + wave * (2 * 32 * 128), lane, row_base, col_of_half(0),
+                               col_of_half(1), result_of_half(0), result_of_half(1));
 }
 
 // Results of the tail tiles: out[tile] = round(sum over parts of ws[tile][part]), fixed order.  One workgroup of
@@ -574,8 +479,8 @@ __global__ __launch_bounds__(256) void fsw_tail_reduce_kernel(GemmParams p) {
     const int m = tc.tm * TM + rem / TN, n = tc.tn * TN + rem % TN;
     if (m >= p.M || n >= p.N) continue;
     u32x2 v;
-    v.x = E::from_float(a.x) | ((unsigned)E::from_float(a.y) << 16);
-    v.y = E::from_float(a.z) | ((unsigned)E::from_float(a.w) << 16);
+    v.x = E::pack2(a.x, a.y);
+    v.y = E::pack2(a.z, a.w);
     unsigned short* out = (unsigned short*)(which == 0 ? p.c0 : p.c1);
     *(u32x2*)(out + (size_t)m * p.ldc + n) = v;
   }

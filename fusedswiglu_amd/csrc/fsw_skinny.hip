@@ -190,8 +190,8 @@ __global__ __launch_bounds__(kSkThreads) void fsw_skinny_forward_kernel(GemmPara
             *(f32x4*)dst = f32x4{v[0], v[1], v[2], v[3]};
           } else {
             u32x2 w;
-            w.x = E::from_float(v[0]) | ((unsigned)E::from_float(v[1]) << 16);
-            w.y = E::from_float(v[2]) | ((unsigned)E::from_float(v[3]) << 16);
+            w.x = E::pack2(v[0], v[1]);
+            w.y = E::pack2(v[2], v[3]);
             *(u32x2*)((unsigned short*)p.c1 + (size_t)m * p.ldc + (size_t)h * p.N + n) = w;
           }
         }

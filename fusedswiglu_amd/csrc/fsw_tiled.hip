@@ -9,8 +9,8 @@ static bool mult8(long long v) { return v > 0 && (v & 7) == 0; }
 static bool al16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 // a per-lane byte offset inside one tile (up to 256 rows) must stay below 2^31
 static bool ld_ok(long long ld) { return mult8(ld) && ld < (1LL << 21); }
-// leading dimension of a result: the kernels keep it in an int and index rows in 64 bits
-static bool ld_out_ok(long long ld) { return mult8(ld) && ld < (1LL << 31); }
+// leading dimension of a result: a wave addresses its up to 128 rows through 32-bit byte offsets from the first
+static bool ld_out_ok(long long ld) { return mult8(ld) && ld < (1LL << 23); }
 static bool dims_ok(const Problem& p) {
   return mult8(p.D) && mult8(p.I) && p.T > 0 && p.T < (1LL << 31) && p.D < (1LL << 31) &&
          p.I < (1LL << 31);

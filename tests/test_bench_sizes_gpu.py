@@ -137,3 +137,64 @@ def test_tail_split_of_the_gradient_gemms(oracle, dtype, out_in, tdi):
     # dx on columns through every tile as well (its tail tiles are tiles of [T, D])
     out2, dx2, dwg2, dwu2 = run_swiglu(dtype, out_in, tx, twg, twu, tdy)
     assert torch.equal(dx, dx2) and torch.equal(dwg, dwg2) and torch.equal(dwu, dwu2)   # fixed summation order
+
+
+# Shapes that take each form of the tiled kernels (eight waves for short reductions, four waves for long ones),
+# with and without edge tiles, a split reduction and a tail split.
+WHOLE_ARRAY_SHAPES = [(4096, 2048, 4352), (2048, 4096, 2048), (512, 2048, 512), (4360, 2056, 4232), (1000, 1032, 776),
+                      (8192, 4096, 5504)]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("out_in", [False, True], ids=["DI", "ID"])
+@pytest.mark.parametrize("tdi", WHOLE_ARRAY_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_every_element_of_every_result(oracle, dtype, out_in, tdi):
+    """The oracle checks above compare slices; a fault confined to a few rows or lanes of a tile could sit between
+    them.  Here every element of out, g, u, dx, dWg and dWu is compared on the GPU with fp32 products of the same
+    16-bit inputs (element-wise bound: a few roundings of the result's magnitude, far below any stale or unconverted
+    value), the oracle confirms the fp32 products on a slice, and a second run must reproduce every bit."""
+    T, D, I = tdi
+    g = torch.Generator(device=DEV).manual_seed(7 * T + I)
+    tx, tdy = randn((T, D), dtype, g), randn((T, I), dtype, g)
+    wshape = (I, D) if out_in else (D, I)
+    twg, twu = randn(wshape, dtype, g, D ** -0.5), randn(wshape, dtype, g, D ** -0.5)
+    def run():
+        out, pg, pu = _launch.fused_swiglu_fwd(tx, twg, twu, dtype, weights_out_in=out_in)
+        dU, dG = _launch.elementwise_backward(tdy, pg, pu, dtype)
+        dx = _launch.fused_input_grad(dG, dU, twg, twu, dtype, weights_out_in=out_in)
+        dwu, dwg = _launch.fused_weight_grad(tx, dU, dG, dtype, weights_out_in=out_in)
+        torch.cuda.synchronize()
+        return out, pg, pu, dG, dU, dx, dwg, dwu
+
+    out, pg, pu, dG, dU, dx, dwg, dwu = run()
+    xf, dyf = tx.float(), tdy.float()
+    wgf, wuf = (twg.float().t(), twu.float().t()) if out_in else (twg.float(), twu.float())   # [D, I]
+    rg, ru = xf @ wgf, xf @ wuf
+    eps = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+
+    def close(name, got, want, scale):
+        err = (got.float() - want).abs()
+        bound = 4 * eps * want.abs() + scale
+        bad = int((~(err <= bound)).sum())   # NaN counts as bad
+        assert bad == 0, f"{name}: {bad} elements outside the bound, worst {err.max().item():.3e}"
+
+    k_fwd, k_dx, k_dw = D ** 0.5, (2 * I) ** 0.5, T ** 0.5
+    close("g", pg, rg, 1e-5 * k_fwd)
+    close("u", pu, ru, 1e-5 * k_fwd)
+    close("out", out, torch.nn.functional.silu(rg) * ru, 1e-5 * k_fwd)
+    # the gradients from the kernels' own (rounded) dG, dU, so that only the GEMM under test contributes
+    dGf, dUf = dG.float(), dU.float()
+    close("dx", dx, dGf @ wgf.t() + dUf @ wuf.t(), 2e-5 * k_dx * dGf.abs().max().item())
+    rdwg, rdwu = xf.t() @ dGf, xf.t() @ dUf
+    if out_in:
+        rdwg, rdwu = rdwg.t(), rdwu.t()
+    close("dWg", dwg, rdwg, 2e-5 * k_dw * dGf.abs().max().item())
+    close("dWu", dwu, rdwu, 2e-5 * k_dw * dUf.abs().max().item())
+    # the fp32 products themselves against the oracle on a few token rows
+    rows = [0, T // 3, T - 1]
+    wg64, wu64 = np64(wgf), np64(wuf)
+    want = oracle.fused_swiglu_fwd(np64(tx[rows]), wg64, wu64)[0]
+    assert oracle.rel_error(np64((torch.nn.functional.silu(rg) * ru)[rows]), want) < 1e-5
+    again = run()
+    for a, b in zip((out, pg, pu, dG, dU, dx, dwg, dwu), again):
+        assert torch.equal(a, b)
