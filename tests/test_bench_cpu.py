@@ -41,3 +41,17 @@ def test_parser_reads_the_table_format(tmp_path):
     assert traffic == {"forward_dual_gemm": 2500 * 1024, "input_grad_dual_gemm": 20 * 1024}
     assert stamp == "0123456789abcdef"
     assert bench.load_profiled_traffic(str(tmp_path / "missing.md")) == ({}, None)
+
+
+def test_no_profiled_read_traffic_below_the_algorithmic_bytes():
+    """Every row of the weight-streaming profile reads at least the bytes the launch must read (both weights and x
+    once): a counter figure below that is an artefact of the summary (e.g. launches of different work averaged
+    together), not a measurement, and must not be committed as traffic."""
+    path = os.path.join(ROOT, "profiles", "skinny_forward_c4_bf16.md")
+    rows = [l for l in open(path) if l.startswith("| fsw_") and "MiB" in l]
+    assert len(rows) >= 8
+    for l in rows:
+        cells = [c.strip() for c in l.strip().strip("|").split("|")]
+        scaled, requests, algorithmic = (float(c.split()[0]) for c in cells[2:5])
+        assert scaled >= 0.995 * algorithmic and requests >= 0.995 * algorithmic, l
+        assert scaled < 1.1 * algorithmic, l
