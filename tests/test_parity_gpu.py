@@ -450,3 +450,25 @@ def test_stream_and_thread_safety(oracle):
     s.synchronize()
     for o in outs:
         assert torch.equal(o, ref)
+
+
+def test_result_leading_dimension_beyond_the_tiled_kernels_limit(oracle):
+    """The tiled kernels address the rows of a wave's results through 32-bit byte offsets, so results whose leading
+    dimension reaches 2^23 elements take the edge kernel (selection code 0) and come out the same."""
+    dtype, T, D, I = torch.bfloat16, 4, 64, 64
+    ldo = 1 << 23
+    L = _abi.lib()
+    assert L.fsw_uses_tiled_kernel(0, 256, D, I, D, I, ldo - 8, I, 16) == 1
+    assert L.fsw_uses_tiled_kernel(0, 256, D, I, D, I, ldo, I, 16) == 0
+    (x, wg, wu, _), (tx, twg, twu, _) = make(oracle, (1, T, D, I), dtype, seed=5)
+    tx = tx[0].contiguous()
+    big = [torch.zeros(T * ldo, device=DEV, dtype=dtype) for _ in range(3)]
+    stream = torch.cuda.current_stream().cuda_stream
+    _abi.check(L.fsw_swiglu_forward(tx.data_ptr(), twg.data_ptr(), twu.data_ptr(), *(b.data_ptr() for b in big),
+                                    T, D, I, D, I, ldo, _abi.DTYPE_BF16, stream))
+    torch.cuda.synchronize()
+    want = oracle.fused_swiglu_fwd(x[0], wg, wu)
+    for b, w in zip(big, want):
+        got = b.view(T, ldo)[:, :I]
+        assert oracle.rel_error(np64(got), w) < 1e-2
+        assert not b.view(T, ldo)[:, I:I + 64].any()      # nothing beyond the rows
