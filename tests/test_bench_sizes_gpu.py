@@ -198,3 +198,53 @@ def test_every_element_of_every_result(oracle, dtype, out_in, tdi):
     again = run()
     for a, b in zip((out, pg, pu, dG, dU, dx, dwg, dwu), again):
         assert torch.equal(a, b)
+
+
+FEW_TOKEN_WHOLE = [(16, 8192, 28672), (64, 4096, 12288), (128, 8192, 28672), (100, 1032, 7176), (256, 8192, 28672),
+                   (200, 4096, 11008)]
+
+
+@pytest.mark.parametrize("out_in", [False, True], ids=["DI", "ID"])
+@pytest.mark.parametrize("tdi", FEW_TOKEN_WHOLE, ids=lambda s: "x".join(map(str, s)))
+def test_every_element_of_the_few_token_forward_and_down_projection(oracle, out_in, tdi):
+    """The weight-streaming kernels (and the tiled kernel with a single row of tiles above 128 tokens) at full
+    width: every element of out, of the down projection y = out W_down and of its input gradient against fp32
+    products of the same inputs on the GPU, the fp32 products against the oracle on one row, and a second run bit
+    for bit."""
+    T, D, I = tdi
+    dtype = torch.bfloat16
+    g = torch.Generator(device=DEV).manual_seed(3 * T + D)
+    tx = randn((T, D), dtype, g)
+    wshape = (I, D) if out_in else (D, I)
+    twg, twu = randn(wshape, dtype, g, D ** -0.5), randn(wshape, dtype, g, D ** -0.5)
+    twd = randn((D, I) if out_in else (I, D), dtype, g, I ** -0.5)
+    tdy = randn((T, D), dtype, g)
+
+    def run():
+        with torch.no_grad():
+            out = _launch.fused_swiglu_fwd(tx, twg, twu, dtype, save_preactivations=False, weights_out_in=out_in)[0]
+            y = _launch.down_proj_forward(out, twd, dtype, weights_out_in=out_in)
+            d_act = _launch.down_proj_input_grad(tdy, twd, dtype, weights_out_in=out_in)
+        torch.cuda.synchronize()
+        return out, y, d_act
+
+    out, y, d_act = run()
+    wgf, wuf = (twg.float().t(), twu.float().t()) if out_in else (twg.float(), twu.float())      # [D, I]
+    wdf = twd.float().t() if out_in else twd.float()                                              # [I, D]
+    xf = tx.float()
+    want = torch.nn.functional.silu(xf @ wgf) * (xf @ wuf)
+    eps = 2.0 ** -8
+
+    def close(name, got, ref, scale):
+        err = (got.float() - ref).abs()
+        bad = int((~(err <= 4 * eps * ref.abs() + scale)).sum())
+        assert bad == 0, f"{name}: {bad} elements outside the bound, worst {err.max().item():.3e}"
+
+    close("out", out, want, 1e-5 * D ** 0.5)
+    close("y", y, out.float() @ wdf, 2e-5 * I ** 0.5 * out.float().abs().max().item())
+    close("d_act", d_act, tdy.float() @ wdf.t(), 2e-5 * D ** 0.5 * tdy.float().abs().max().item())
+    row = [T // 2]
+    o_row = oracle.fused_swiglu_fwd(np64(tx[row]), np64(wgf), np64(wuf))[0]
+    assert oracle.rel_error(np64(want[row]), o_row) < 1e-5
+    for a, b in zip((out, y, d_act), run()):
+        assert torch.equal(a, b)
