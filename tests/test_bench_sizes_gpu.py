@@ -163,10 +163,12 @@ def test_every_element_of_every_result(oracle, dtype, out_in, tdi):
         dU, dG = _launch.elementwise_backward(tdy, pg, pu, dtype)
         dx = _launch.fused_input_grad(dG, dU, twg, twu, dtype, weights_out_in=out_in)
         dwu, dwg = _launch.fused_weight_grad(tx, dU, dG, dtype, weights_out_in=out_in)
+        # the gating gradient again, from x and the weights (forward kernel with the gating-gradient epilogue)
+        rU, rG = _launch.gating_grad_recompute(tdy, tx, twg, twu, dtype, weights_out_in=out_in)
         torch.cuda.synchronize()
-        return out, pg, pu, dG, dU, dx, dwg, dwu
+        return out, pg, pu, dG, dU, dx, dwg, dwu, rU, rG
 
-    out, pg, pu, dG, dU, dx, dwg, dwu = run()
+    out, pg, pu, dG, dU, dx, dwg, dwu, rU, rG = run()
     xf, dyf = tx.float(), tdy.float()
     wgf, wuf = (twg.float().t(), twu.float().t()) if out_in else (twg.float(), twu.float())   # [D, I]
     rg, ru = xf @ wgf, xf @ wuf
@@ -182,6 +184,9 @@ def test_every_element_of_every_result(oracle, dtype, out_in, tdi):
     close("g", pg, rg, 1e-5 * k_fwd)
     close("u", pu, ru, 1e-5 * k_fwd)
     close("out", out, torch.nn.functional.silu(rg) * ru, 1e-5 * k_fwd)
+    sg = torch.sigmoid(rg)
+    close("recomputed dU", rU, dyf * rg * sg, 1e-5 * k_fwd)
+    close("recomputed dG", rG, dyf * ru * (sg + rg * sg * (1 - sg)), 4e-5 * k_fwd)
     # the gradients from the kernels' own (rounded) dG, dU, so that only the GEMM under test contributes
     dGf, dUf = dG.float(), dU.float()
     close("dx", dx, dGf @ wgf.t() + dUf @ wuf.t(), 2e-5 * k_dx * dGf.abs().max().item())
@@ -196,7 +201,7 @@ def test_every_element_of_every_result(oracle, dtype, out_in, tdi):
     want = oracle.fused_swiglu_fwd(np64(tx[rows]), wg64, wu64)[0]
     assert oracle.rel_error(np64((torch.nn.functional.silu(rg) * ru)[rows]), want) < 1e-5
     again = run()
-    for a, b in zip((out, pg, pu, dG, dU, dx, dwg, dwu), again):
+    for a, b in zip((out, pg, pu, dG, dU, dx, dwg, dwu, rU, rG), again):
         assert torch.equal(a, b)
 
 
