@@ -150,11 +150,7 @@ static hipError_t launch(int dtype, GemmParams g, hipStream_t s, void* ws = null
   const bool w4_fits = (Cfg<MODE>::kAKc || (long long)g.K * g.lda * 2 < (1LL << 31)) &&
                        (Cfg<MODE>::kBKc || (long long)g.K * g.ldb * 2 < (1LL << 31));
   const int steps_per_workgroup = pl.splits > 1 ? pl.steps_per_split : steps;
-#if defined(FSW_FORCE_WAVES)
-  const bool four_waves = w4_fits && FSW_FORCE_WAVES == 4;
-#else
   const bool four_waves = w4_fits && steps_per_workgroup >= (Cfg<MODE>::kForward ? 96 : 64);
-#endif
   long long grid4 = grid;
   if constexpr (!Cfg<MODE>::kForward) {
     const TailPlan tp = plan_tail(tiles, steps);
