@@ -41,6 +41,7 @@ EXPORTED_SYMBOLS = (
     "fsw_input_grad",
     "fsw_input_grad_noalloc",
     "fsw_weight_grad",
+    "fsw_swiglu_backward",
     "fsw_down_proj_forward",
     "fsw_down_proj_input_grad",
     "fsw_down_proj_weight_grad",
@@ -115,6 +116,8 @@ def lib() -> ctypes.CDLL:
         L.fsw_input_grad_noalloc.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, vp]
         L.fsw_weight_grad.restype = ci
         L.fsw_weight_grad.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, i64, ci, vp]
+        L.fsw_swiglu_backward.restype = ci
+        L.fsw_swiglu_backward.argtypes = [vp] * 11 + [i64] * 7 + [vp, i64, ci, vp]
         for name in ("fsw_down_proj_forward", "fsw_down_proj_input_grad", "fsw_down_proj_weight_grad"):
             getattr(L, name).restype = ci
             getattr(L, name).argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, i64, ci, vp]

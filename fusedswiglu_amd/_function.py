@@ -34,20 +34,14 @@ def forward_training(ctx, kernels, input, weight_gate, weight_up):
 
 def backward(ctx, kernels, grad_output):
     """fused_swiglu/swiglu.py:34-58.  Returns (grad_input, grad_weight_gate, grad_weight_up).
-    Three launches: gating gradient, input-gradient dual GEMM, weight-gradient dual GEMM (reduced
-    over all tokens, so the reference's per-batch partials and `unbroadcast` sum disappear).
+    One library call, three launches: gating gradient, input-gradient dual GEMM, weight-gradient dual GEMM
+    (reduced over all tokens, so the reference's per-batch partials and `unbroadcast` sum disappear).
     Gradients nobody asked for (ctx.needs_input_grad) are skipped."""
     input, weight_gate, weight_up, xw_gate, xw_up = ctx.saved_tensors
     if grad_output.dtype != xw_gate.dtype:
         grad_output = grad_output.to(xw_gate.dtype)
-    grad_xw_up, grad_xw_gate = kernels.elementwise_backward(grad_output, xw_gate, xw_up)
-    grad_input = grad_weight_gate = grad_weight_up = None
-    if ctx.needs_input_grad[0]:
-        grad_input = kernels.fused_input_grad(grad_xw_gate, grad_xw_up, weight_gate, weight_up)
-    if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
-        grad_weight_up, grad_weight_gate = kernels.fused_weight_grad(input, grad_xw_up, grad_xw_gate)
-        if not ctx.needs_input_grad[1]:
-            grad_weight_gate = None
-        if not ctx.needs_input_grad[2]:
-            grad_weight_up = None
-    return grad_input, grad_weight_gate, grad_weight_up
+    need = ctx.needs_input_grad
+    grad_input, grad_weight_gate, grad_weight_up = kernels.swiglu_backward(
+        grad_output, input, weight_gate, weight_up, xw_gate, xw_up,
+        need_input_grad=need[0], need_weight_grad=need[1] or need[2])
+    return grad_input, grad_weight_gate if need[1] else None, grad_weight_up if need[2] else None

@@ -224,22 +224,30 @@ int fsw_input_grad(const void* grad_xw_gate, const void* grad_xw_up, const void*
                             workspace, workspace_bytes, dtype, stream);
 }
 
+static int check_weight_grad_args(const char* fn, const void* x, const void* grad_xw_up, const void* grad_xw_gate,
+                                  void* grad_w_up, void* grad_w_gate, int64_t T, int64_t D, int64_t I, int64_t ldx,
+                                  int64_t ldo, int64_t ld_dw, int dtype) {
+  if (!x || !grad_xw_up || !grad_xw_gate || !grad_w_up || !grad_w_gate)
+    return fail(FSW_ERR_NULL_POINTER, "%s: all five arrays must be non-null", fn);
+  if (!dtype_ok(dtype)) return fail(FSW_ERR_BAD_DTYPE, "%s: dtype %d is neither bf16 (0) nor fp16 (1)", fn, dtype);
+  if (int e = check_dims(fn, T, D, I)) return e;
+  if (int e = check_ld(fn, "ldx", ldx, D)) return e;
+  if (int e = check_ld(fn, "ldo", ldo, I)) return e;
+  if (int e = check_ld(fn, "ld_dw", ld_dw, out_in_of(dtype) ? D : I)) return e;
+  if (!al2(x) || !al2(grad_xw_up) || !al2(grad_xw_gate) || !al2(grad_w_up) || !al2(grad_w_gate))
+    return fail(FSW_ERR_ALIGNMENT, "%s: pointers must be 2-byte aligned", fn);
+  return FSW_OK;
+}
+
 int fsw_weight_grad(const void* x, const void* grad_xw_up, const void* grad_xw_gate,
                     void* grad_w_up, void* grad_w_gate, int64_t T, int64_t D, int64_t I,
                     int64_t ldx, int64_t ldo, int64_t ld_dw, void* workspace, int64_t workspace_bytes,
                     int dtype, void* stream) {
   const char* fn = "fsw_weight_grad";
-  if (!x || !grad_xw_up || !grad_xw_gate || !grad_w_up || !grad_w_gate)
-    return fail(FSW_ERR_NULL_POINTER, "%s: all five arrays must be non-null", fn);
-  if (!dtype_ok(dtype)) return fail(FSW_ERR_BAD_DTYPE, "%s: dtype %d is neither bf16 (0) nor fp16 (1)", fn, dtype);
-  if (int e = check_dims(fn, T, D, I)) return e;
+  if (int e = check_weight_grad_args(fn, x, grad_xw_up, grad_xw_gate, grad_w_up, grad_w_gate, T, D, I, ldx, ldo, ld_dw, dtype))
+    return e;
   const bool oi = out_in_of(dtype);
   dtype = elem_of(dtype);
-  if (int e = check_ld(fn, "ldx", ldx, D)) return e;
-  if (int e = check_ld(fn, "ldo", ldo, I)) return e;
-  if (int e = check_ld(fn, "ld_dw", ld_dw, oi ? D : I)) return e;
-  if (!al2(x) || !al2(grad_xw_up) || !al2(grad_xw_gate) || !al2(grad_w_up) || !al2(grad_w_gate))
-    return fail(FSW_ERR_ALIGNMENT, "%s: pointers must be 2-byte aligned", fn);
   fsw::Problem p{};
   p.x = x; p.dG = grad_xw_gate; p.dU = grad_xw_up; p.dWg = grad_w_gate; p.dWu = grad_w_up;
   p.T = T; p.D = D; p.I = I; p.ldx = ldx; p.ldo = ldo; p.lddw = ld_dw; p.w_out_in = oi;
@@ -249,6 +257,42 @@ int fsw_weight_grad(const void* x, const void* grad_xw_up, const void* grad_xw_g
     return launched(fn, fsw::launch_weight_grad_fast(dtype, p, s, ws_ok ? workspace : nullptr, ws_ok ? workspace_bytes : 0));
   }
   return launched(fn, fsw::launch_weight_grad_generic(dtype, p, s));
+}
+
+int fsw_swiglu_backward(const void* grad_out, const void* xw_gate, const void* xw_up, const void* x,
+                        const void* w_gate, const void* w_up, void* grad_xw_gate, void* grad_xw_up, void* grad_x,
+                        void* grad_w_gate, void* grad_w_up, int64_t T, int64_t D, int64_t I, int64_t ldx,
+                        int64_t ldw, int64_t ld_dx, int64_t ld_dw, void* workspace, int64_t workspace_bytes,
+                        int dtype, void* stream) {
+  const char* fn = "fsw_swiglu_backward";
+  if ((grad_w_gate == nullptr) != (grad_w_up == nullptr))
+    return fail(FSW_ERR_NULL_POINTER, "%s: grad_w_gate and grad_w_up must both be given or both be null", fn);
+  if (grad_x && (!w_gate || !w_up)) return fail(FSW_ERR_NULL_POINTER, "%s: grad_x needs w_gate and w_up", fn);
+  if (grad_w_gate && !x) return fail(FSW_ERR_NULL_POINTER, "%s: the weight gradients need x", fn);
+  // everything is validated before the first launch: a call that fails has enqueued nothing
+  if (!grad_out || !xw_gate || !xw_up || !grad_xw_gate || !grad_xw_up)
+    return fail(FSW_ERR_NULL_POINTER, "%s: grad_out, xw_gate, xw_up, grad_xw_gate and grad_xw_up must be non-null", fn);
+  if (!dtype_ok(dtype)) return fail(FSW_ERR_BAD_DTYPE, "%s: dtype %d is neither bf16 (0) nor fp16 (1)", fn, dtype);
+  if (int e = check_dims(fn, T, D, I)) return e;
+  if (!al2(grad_out) || !al2(xw_gate) || !al2(xw_up))
+    return fail(FSW_ERR_ALIGNMENT, "%s: pointers must be 2-byte aligned", fn);
+  if (grad_x)
+    if (int e = check_input_grad_args(fn, grad_xw_gate, grad_xw_up, w_gate, w_up, grad_x, T, D, I, I, ldw, ld_dx, dtype))
+      return e;
+  if (grad_w_gate)
+    if (int e = check_weight_grad_args(fn, x, grad_xw_up, grad_xw_gate, grad_w_up, grad_w_gate, T, D, I, ldx, I, ld_dw, dtype))
+      return e;
+  if (int e = fsw_elementwise_backward(grad_out, xw_gate, xw_up, grad_xw_up, grad_xw_gate, T * I, elem_of(dtype), stream))
+    return e;
+  if (grad_x)
+    if (int e = fsw_input_grad(grad_xw_gate, grad_xw_up, w_gate, w_up, grad_x, T, D, I, I, ldw, ld_dx, workspace,
+                               workspace_bytes, dtype, stream))
+      return e;
+  if (grad_w_gate)
+    if (int e = fsw_weight_grad(x, grad_xw_up, grad_xw_gate, grad_w_up, grad_w_gate, T, D, I, ldx, I, ld_dw, workspace,
+                                workspace_bytes, dtype, stream))
+      return e;
+  return FSW_OK;
 }
 
 // ---- the down projection that follows the SwiGLU: three plain GEMMs on the same tiled kernels ----

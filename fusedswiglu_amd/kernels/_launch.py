@@ -36,9 +36,11 @@ def _require(cond: bool, msg: str) -> None:
 
 def _check_device(*tensors: torch.Tensor) -> torch.device:
     dev = tensors[0].device
-    _require(dev.type == "cuda", f"fused SwiGLU needs tensors on a HIP GPU, got device '{dev}'")
+    if dev.type != "cuda":
+        raise ShapeError(f"fused SwiGLU needs tensors on a HIP GPU, got device '{dev}'")
     for t in tensors[1:]:
-        _require(t.device == dev, f"all tensors must be on the same device ({t.device} vs {dev})")
+        if t.device != dev:
+            raise ShapeError(f"all tensors must be on the same device ({t.device} vs {dev})")
     return dev
 
 
@@ -73,6 +75,8 @@ class _on_device:
 
 def _rows(t: torch.Tensor) -> torch.Tensor:
     """2-D [rows, cols] view with unit inner stride (copies only if it must)."""
+    if t.ndim == 2 and t.stride(1) == 1 and (t.shape[0] <= 1 or t.stride(0) >= t.shape[1]):
+        return t
     t2 = t.reshape(-1, t.shape[-1])
     if t2.stride(-1) != 1 or (t2.shape[0] > 1 and t2.stride(0) < t2.shape[1]):
         t2 = t2.contiguous()
@@ -110,13 +114,16 @@ def fused_swiglu_fwd(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, 
     _require(x.ndim >= 2 and w_up.ndim == 2 and w_gate.ndim == 2,
              "Incorrect number of dimensions for LHS or RHS")
     D, I = _weight_dims(w_up, weights_out_in)
-    _require(x.shape[-1] == D,
-             f"Dimension mismatch. Expected x.shape[-1] ({x.shape[-1]}) to be equal to "
-             f"w_up.shape[{1 if weights_out_in else 0}] ({D})")
+    # (the messages are only built when a check fails: this runs once per training step)
+    if x.shape[-1] != D:
+        raise ShapeError(f"Dimension mismatch. Expected x.shape[-1] ({x.shape[-1]}) to be equal to "
+                         f"w_up.shape[{1 if weights_out_in else 0}] ({D})")
     _require(w_up.shape == w_gate.shape, "Expected both weight matrices to have same shape")
-    _require(x.dtype == dtype and w_gate.dtype == dtype and w_up.dtype == dtype,
-             f"Expected {dtype} inputs and weights, got {x.dtype}, {w_gate.dtype}, {w_up.dtype}")
-    dev = _check_device(x, w_gate, w_up)
+    if not (x.dtype == dtype and w_gate.dtype == dtype and w_up.dtype == dtype):
+        raise ShapeError(f"Expected {dtype} inputs and weights, got {x.dtype}, {w_gate.dtype}, {w_up.dtype}")
+    dev = x.device
+    if dev.type != "cuda" or w_gate.device != dev or w_up.device != dev:
+        _check_device(x, w_gate, w_up)
     _require(x.numel() > 0 and I > 0, "empty input")
     x2, wg, wu = _rows(x), _rows(w_gate), _rows(w_up)
     if _ld(wg) != _ld(wu):
@@ -212,6 +219,53 @@ def fused_input_grad(grad_xw_gate: torch.Tensor, grad_xw_up: torch.Tensor, w_gat
             T, D, I, _ld(dg), _ld(wg), D, ws.data_ptr() if ws is not None else None, ws_bytes,
             _code(dtype, weights_out_in), _stream_ptr(dev)))
     return grad_x
+
+
+def swiglu_backward(grad_output: torch.Tensor, x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor,
+                    xw_gate: torch.Tensor, xw_up: torch.Tensor, dtype: torch.dtype, need_input_grad: bool = True,
+                    need_weight_grad: bool = True, weights_out_in: bool = False
+                    ) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor], Optional[torch.Tensor]]:
+    """(grad_x, grad_w_gate, grad_w_up) of fused_swiglu/swiglu.py:34-58 in ONE library call: the gating gradient,
+    then the input-gradient and weight-gradient GEMMs that were asked for.  Same kernels, same results as
+    elementwise_backward + fused_input_grad + fused_weight_grad; two trips through ctypes and their argument checks
+    fewer, which is most of a training step's host time when d_model is small."""
+    D, I = _weight_dims(w_gate, weights_out_in)
+    if not (x.ndim >= 2 and w_gate.ndim == 2 and w_gate.shape == w_up.shape and x.shape[-1] == D
+            and xw_gate.shape == xw_up.shape == grad_output.shape and tuple(grad_output.shape) == tuple(x.shape[:-1]) + (I,)):
+        raise ShapeError(f"swiglu_backward: shapes do not fit: x {tuple(x.shape)}, weights {tuple(w_gate.shape)} / "
+                         f"{tuple(w_up.shape)}, pre-activations {tuple(xw_gate.shape)} / {tuple(xw_up.shape)}, "
+                         f"grad_output {tuple(grad_output.shape)}")
+    if not (x.dtype == w_gate.dtype == w_up.dtype == xw_gate.dtype == xw_up.dtype == grad_output.dtype == dtype):
+        raise ShapeError(f"Expected {dtype} tensors")
+    dev = x.device
+    if dev.type != "cuda" or not (w_gate.device == w_up.device == xw_gate.device == xw_up.device == grad_output.device == dev):
+        _check_device(x, w_gate, w_up, xw_gate, xw_up, grad_output)   # raises with the offending pair
+    if x.numel() == 0 or I == 0:
+        raise ShapeError("empty input")
+    x2, wg, wu = _rows(x), _rows(w_gate), _rows(w_up)
+    if _ld(wg) != _ld(wu):
+        wg, wu = wg.contiguous(), wu.contiguous()
+    # the gating gradient indexes flat, dense arrays
+    dout, g, u = grad_output.contiguous(), xw_gate.contiguous(), xw_up.contiguous()
+    T = x2.shape[0]
+    grad_xw_gate, grad_xw_up = torch.empty_like(dout), torch.empty_like(dout)
+    grad_x = torch.empty(x.shape, device=dev, dtype=dtype) if need_input_grad else None
+    grad_w_gate = torch.empty(w_gate.shape, device=dev, dtype=dtype) if need_weight_grad else None
+    grad_w_up = torch.empty(w_up.shape, device=dev, dtype=dtype) if need_weight_grad else None
+    with _on_device(dev):
+        L = _abi.lib()
+        flag = _abi.WEIGHTS_OUT_IN if weights_out_in else 0
+        nbytes = max(int(L.fsw_workspace_bytes(_abi.STEP_INPUT_GRAD | flag, T, D, I)) if need_input_grad else 0,
+                     int(L.fsw_workspace_bytes(_abi.STEP_WEIGHT_GRAD | flag, T, D, I)) if need_weight_grad else 0)
+        ws = torch.empty(nbytes, device=dev, dtype=torch.uint8) if nbytes > 0 else None
+        ld_dw = w_gate.shape[1]
+        _abi.check(L.fsw_swiglu_backward(
+            dout.data_ptr(), g.data_ptr(), u.data_ptr(), x2.data_ptr(), wg.data_ptr(), wu.data_ptr(),
+            grad_xw_gate.data_ptr(), grad_xw_up.data_ptr(), grad_x.data_ptr() if need_input_grad else None,
+            grad_w_gate.data_ptr() if need_weight_grad else None, grad_w_up.data_ptr() if need_weight_grad else None,
+            T, D, I, _ld(x2), _ld(wg), D, ld_dw, ws.data_ptr() if ws is not None else None, nbytes,
+            _code(dtype, weights_out_in), _stream_ptr(dev)))
+    return grad_x, grad_w_gate, grad_w_up
 
 
 def fused_weight_grad(x: torch.Tensor, grad_xw_up: torch.Tensor, grad_xw_gate: torch.Tensor,

@@ -13,4 +13,5 @@ elementwise_backward = partial(_launch.elementwise_backward, dtype=_DT)
 gating_grad_recompute = partial(_launch.gating_grad_recompute, dtype=_DT)
 fused_input_grad = partial(_launch.fused_input_grad, dtype=_DT)
 fused_weight_grad = partial(_launch.fused_weight_grad, dtype=_DT)
+swiglu_backward = partial(_launch.swiglu_backward, dtype=_DT)
 fused_bmm = partial(_launch.fused_bmm, dtype=_DT)

@@ -42,11 +42,12 @@ extern "C" {
 #endif
 
 /* major*10000 + minor*100 + patch.
+ * 0.4.0: fsw_swiglu_backward (the three backward steps in one call).
  * 0.3.0: FSW_WEIGHTS_OUT_IN, the fsw_down_proj_* entry points, fsw_input_grad_noalloc and status 7,
  *        fsw_uses_tiled_kernel answers 2 for the weight-streaming kernels and knows steps 4 / 5 / 6,
  *        fsw_workspace_bytes may ask for up to 64 MiB for large gradient GEMMs (tail split).
  * 0.2.0: fsw_gating_grad_recompute. */
-#define FSW_VERSION 300
+#define FSW_VERSION 400
 
 enum { FSW_DTYPE_BF16 = 0, FSW_DTYPE_FP16 = 1 };
 /* May be OR-ed into any `dtype` argument (and into the `step` of fsw_workspace_bytes): the weights of the
@@ -171,6 +172,23 @@ FSW_API int fsw_weight_grad(const void* x, const void* grad_xw_up, const void* g
                     void* grad_w_up, void* grad_w_gate, int64_t T, int64_t D, int64_t I,
                     int64_t ldx, int64_t ldo, int64_t ld_dw, void* workspace, int64_t workspace_bytes,
                     int dtype, void* stream);
+
+/*
+ * The whole backward of the path in one call: the body of FusedSwiGLU.backward (fused_swiglu/swiglu.py:34-58).
+ * Exactly fsw_elementwise_backward, then fsw_input_grad (if grad_x is given), then fsw_weight_grad (if the two weight
+ * gradients are given), enqueued on `stream` in that order - for hosts where three calls through a foreign-function
+ * interface cost more than the small kernels they launch.
+ *   grad_out, xw_gate, xw_up, grad_xw_gate, grad_xw_up [T,I] dense (leading dimension I)
+ *   x [T,D] (ldx)   w_gate, w_up (ldw)   grad_x [T,D] (ld_dx)   grad_w_gate, grad_w_up (ld_dw)
+ * grad_xw_gate and grad_xw_up are results too (the gating gradients), always written.  grad_x may be NULL, and
+ * grad_w_gate / grad_w_up both NULL: that gradient is skipped (ctx.needs_input_grad).  `workspace` is used by the
+ * two GEMMs one after the other: the larger of fsw_workspace_bytes(1, ...) and fsw_workspace_bytes(2, ...) serves both.
+ */
+FSW_API int fsw_swiglu_backward(const void* grad_out, const void* xw_gate, const void* xw_up, const void* x,
+                        const void* w_gate, const void* w_up, void* grad_xw_gate, void* grad_xw_up, void* grad_x,
+                        void* grad_w_gate, void* grad_w_up, int64_t T, int64_t D, int64_t I, int64_t ldx,
+                        int64_t ldw, int64_t ld_dx, int64_t ld_dw, void* workspace, int64_t workspace_bytes,
+                        int dtype, void* stream);
 
 /*
  * The down projection that follows the SwiGLU in an MLP block, y = act W_down, and its two gradients, on the

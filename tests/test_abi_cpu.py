@@ -44,7 +44,7 @@ def test_header_symbols_all_exported(L):
         assert getattr(L, name) is not None
     header = open(os.path.join(ROOT, "include", "fusedswiglu.h")).read()
     m = re.search(r"#define FSW_VERSION (\d+)", header)
-    assert L.fsw_version() == int(m.group(1)) == 300   # 0.3.0: layouts, down projection, no-allocation entry point
+    assert L.fsw_version() == int(m.group(1)) == 400   # 0.4.0: the backward in one call
     assert "probe" not in header and "force_edge" not in header
     bench = _declared("fusedswiglu_bench.h")
     assert bench == set(_abi.BENCH_SYMBOLS) == _exported(_abi.BENCH_LIBRARY_PATH)
@@ -89,6 +89,19 @@ def test_backward_validation(L):
     assert rc(P, P, P, P, P, P, 8, 0, 8, 8, 8, 8, 0, None) == 3
     assert rc(P, P, P, P, P, P, 8, 8, 16, 8, 16, 8, 0, None) == 4  # ldo < I
     assert rc(P, P, P, ctypes.c_void_p(0x1001), P, P, 8, 8, 8, 8, 8, 8, 0, None) == 5
+    # the backward in one call validates all three steps before it launches the first
+    bw = L.fsw_swiglu_backward
+    ok_dims = (8, 8, 8, 8, 8, 8, 8)                                    # T, D, I, ldx, ldw, ld_dx, ld_dw
+    assert bw(P, P, None, P, P, P, P, P, P, P, P, *ok_dims, None, 0, 0, None) == 1          # no xw_up
+    assert bw(P, P, P, P, P, P, P, P, P, P, None, *ok_dims, None, 0, 0, None) == 1          # one weight gradient only
+    assert bw(P, P, P, P, None, P, P, P, P, P, P, *ok_dims, None, 0, 0, None) == 1          # grad_x without w_gate
+    assert bw(P, P, P, None, P, P, P, P, None, P, P, *ok_dims, None, 0, 0, None) == 1       # weight gradients without x
+    assert bw(P, P, P, P, P, P, P, P, P, P, P, 8, 8, 8, 8, 8, 4, 8, None, 0, 0, None) == 4  # ld_dx < D
+    assert bw(P, P, P, P, P, P, P, P, P, P, P, 8, 8, 16, 8, 16, 8, 8, None, 0, 0, None) == 4  # ld_dw < I
+    assert bw(P, P, P, P, P, P, P, P, P, P, P, 8, 16, 8, 8, 8, 16, 8, None, 0, 0, None) == 4  # ldx < D
+    assert bw(P, P, P, P, P, P, P, P, P, P, P, 0, 8, 8, 8, 8, 8, 8, None, 0, 0, None) == 3
+    assert bw(P, P, P, P, P, P, P, P, P, P, P, *ok_dims, None, 0, 4, None) == 2
+    assert bw(ctypes.c_void_p(0x1001), P, P, P, P, P, P, P, P, P, P, *ok_dims, None, 0, 0, None) == 5
     dx = L.fsw_input_grad
     assert dx(P, P, P, P, None, 8, 8, 8, 8, 8, 8, None, 0, 0, None) == 1
     assert dx(P, P, P, P, P, 8, 8, 8, 8, 8, 4, None, 0, 0, None) == 4  # ld_dx < D

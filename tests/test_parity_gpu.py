@@ -472,3 +472,35 @@ def test_result_leading_dimension_beyond_the_tiled_kernels_limit(oracle):
         got = b.view(T, ldo)[:, :I]
         assert oracle.rel_error(np64(got), w) < 1e-2
         assert not b.view(T, ldo)[:, I:I + 64].any()      # nothing beyond the rows
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("out_in", [False, True], ids=["DI", "ID"])
+@pytest.mark.parametrize("shape", [(2, 136, 264, 520), (1, 2048, 256, 768), (3, 50, 72, 65), (1, 4096, 2048, 1024)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_backward_in_one_call_equals_the_three_steps(oracle, dtype, out_in, shape):
+    """fsw_swiglu_backward (fused_swiglu/swiglu.py:34-58 as one library call) enqueues the same three kernels as
+    elementwise_backward + fused_input_grad + fused_weight_grad: identical bits, against the oracle, and with
+    either gradient switched off."""
+    from fusedswiglu_amd.kernels import _launch
+    (x, wg, wu, dy), (tx, twg, twu, tdy) = make(oracle, shape, dtype, seed=31)
+    if out_in:
+        twg, twu = twg.t().contiguous(), twu.t().contiguous()
+    _, tg, tu = _launch.fused_swiglu_fwd(tx, twg, twu, dtype, weights_out_in=out_in)
+    dU, dG = _launch.elementwise_backward(tdy, tg, tu, dtype)
+    dx3 = _launch.fused_input_grad(dG, dU, twg, twu, dtype, weights_out_in=out_in)
+    dwu3, dwg3 = _launch.fused_weight_grad(tx, dU, dG, dtype, weights_out_in=out_in)
+    dx1, dwg1, dwu1 = _launch.swiglu_backward(tdy, tx, twg, twu, tg, tu, dtype, weights_out_in=out_in)
+    torch.cuda.synchronize()
+    assert dx1.shape == tx.shape and dwg1.shape == twg.shape and dwu1.shape == twu.shape
+    assert torch.equal(dx1, dx3) and torch.equal(dwg1, dwg3) and torch.equal(dwu1, dwu3)
+    o_dx, o_dwg, o_dwu = oracle.swiglu_backward(x, wg, wu, dy)
+    tol = TOL[dtype]
+    assert oracle.rel_error(np64(dx1), o_dx) < tol
+    assert oracle.rel_error(np64(dwg1.t() if out_in else dwg1), o_dwg) < tol
+    assert oracle.rel_error(np64(dwu1.t() if out_in else dwu1), o_dwu) < tol
+    only_x = _launch.swiglu_backward(tdy, tx, twg, twu, tg, tu, dtype, need_weight_grad=False, weights_out_in=out_in)
+    only_w = _launch.swiglu_backward(tdy, tx, twg, twu, tg, tu, dtype, need_input_grad=False, weights_out_in=out_in)
+    torch.cuda.synchronize()
+    assert only_x[1] is None and only_x[2] is None and torch.equal(only_x[0], dx3)
+    assert only_w[0] is None and torch.equal(only_w[1], dwg3) and torch.equal(only_w[2], dwu3)
