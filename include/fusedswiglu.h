@@ -175,8 +175,8 @@ FSW_API int fsw_weight_grad(const void* x, const void* grad_xw_up, const void* g
 
 /*
  * The whole backward of the path in one call: the body of FusedSwiGLU.backward (fused_swiglu/swiglu.py:34-58).
- * Exactly fsw_elementwise_backward, then fsw_input_grad (if grad_x is given), then fsw_weight_grad (if the two weight
- * gradients are given), enqueued on `stream` in that order - for hosts where three calls through a foreign-function
+ * Exactly fsw_elementwise_backward, then fsw_weight_grad (if the two weight gradients are given), then fsw_input_grad
+ * (if grad_x is given), enqueued on `stream` in that order - for hosts where three calls through a foreign-function
  * interface cost more than the small kernels they launch.
  *   grad_out, xw_gate, xw_up, grad_xw_gate, grad_xw_up [T,I] dense (leading dimension I)
  *   x [T,D] (ldx)   w_gate, w_up (ldw)   grad_x [T,D] (ld_dx)   grad_w_gate, grad_w_up (ld_dw)
