@@ -84,13 +84,18 @@ def swiglu_backward(grad_out: Tensor, x: Tensor, w_gate: Tensor, w_up: Tensor, x
     oi = weights_out_in
     if grad_out.dtype != dtype:
         grad_out = grad_out.to(dtype)
+    e = _empty(x)
+    if xw_gate.numel() != 0 and not packed:
+        # the common case in one library call (gating gradient, weight gradient, input gradient)
+        dx, dw_gate, dw_up = _launch.swiglu_backward(grad_out, x, w_gate, w_up, xw_gate, xw_up, dtype, need_input_grad=need_x,
+                                                     need_weight_grad=need_w_gate or need_w_up, weights_out_in=oi)
+        return (dx if dx is not None else e, dw_gate if need_w_gate else e.clone(), dw_up if need_w_up else e.clone())
     if xw_gate.numel() == 0:
         d_up, d_gate = _launch.gating_grad_recompute(grad_out, x, w_gate, w_up, dtype, weights_out_in=oi)
     else:
         d_up, d_gate = _launch.elementwise_backward(grad_out, xw_gate, xw_up, dtype)
     dx = dw_gate = dw_up = None
-    if need_x:
-        dx = _launch.fused_input_grad(d_gate, d_up, w_gate, w_up, dtype, weights_out_in=oi)
+    # the weight gradient first: the input gradient then finds d_gate and d_up in the memory-side cache
     if need_w_gate or need_w_up:
         if packed and oi:
             I, D = w_gate.shape
@@ -106,7 +111,8 @@ def swiglu_backward(grad_out: Tensor, x: Tensor, w_gate: Tensor, w_up: Tensor, x
                 dw_gate = None
             if not need_w_up:
                 dw_up = None
-    e = _empty(x)
+    if need_x:
+        dx = _launch.fused_input_grad(d_gate, d_up, w_gate, w_up, dtype, weights_out_in=oi)
     return (dx if dx is not None else e, dw_gate if dw_gate is not None else e.clone(),
             dw_up if dw_up is not None else e.clone())
 
