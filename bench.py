@@ -269,7 +269,12 @@ def main():
             ceil[name] = round(fl.value / ms / 1e9, 1)
         # the 16x16x32 instruction the tiled kernels use (mix 0 of the probe: no data movement beside it)
         window = torch.empty(8 << 20, device=dev, dtype=torch.uint8).fill_(60)
-        for name, mix in (("mfma_16x16x32_normal_operands_tflops", 0),):
+        # mix 1: the tiled kernels' LDS reads and direct loads beside the MFMAs; mix 5: the same with the
+        # weight-side fragments formed by the gating-gradient arithmetic instead of held in registers - what the
+        # matrix cores would deliver to a weight-gradient GEMM that absorbed the gating-gradient kernel
+        for name, mix in (("mfma_16x16x32_normal_operands_tflops", 0),
+                          ("mfma_16x16x32_with_tile_data_movement_tflops", 1),
+                          ("mfma_16x16x32_with_gating_gradient_in_operand_path_tflops", 5)):
             fl = ctypes.c_double(0.0)
             run = lambda: _abi.check(_abi.bench_lib().fsw_probe_mfma_mix(mix, 10000, 2 * ncu, p(window), window.numel(), p(sink), stream, ctypes.byref(fl)))  # noqa: E731
             ms = gpu_time_ms(run, iters=3, warmup=1)

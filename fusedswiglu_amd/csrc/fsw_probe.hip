@@ -48,14 +48,19 @@ __global__ __launch_bounds__(512) void probe_mfma_kernel(float* sink, int iters,
 // per wave, the loads hitting L2 (the 32 CUs of an XCD walk one 8 MiB window).  LDS values are consumed
 // one iteration after they were read, so nothing ever waits for fresh data: what this loop sustains is
 // what the matrix cores deliver while that much data moves beside them.
-template <int NR, int ND>
+// GATING (needs NR == 3): the weight-side fragment of the NEXT 8 MFMAs is not held in registers but formed from
+// the three values just read from LDS, taken as dout, g, u (bf16 ~N(0,1)): four gating gradients dG, dU per lane
+// and 8 MFMAs, which is what a 128x128 wave tile of the weight-gradient GEMM would have to compute if the
+// gating-gradient kernel were folded into its operand path (8 fragments of 8 values per 64 MFMAs).
+template <int NR, int ND, bool GATING = false>
 __global__ __launch_bounds__(512) void probe_mfma_mix_kernel(const char* src, unsigned src_bytes, float* sink, int iters) {
+  static_assert(!GATING || NR == 3, "the gating mix takes dout, g, u from the three reads");
   __shared__ __attribute__((aligned(1024))) char smem[64 * 1024];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   for (int i = tid; i < 64 * 1024 / 16; i += 512) {
     u32x4 v;
-    for (int e = 0; e < 4; e++) v[e] = __float_as_uint(probe_normal(i * 4 + e, 7));
+    for (int e = 0; e < 4; e++) v[e] = BF16::pack2(probe_normal(i * 8 + 2 * e, 7), probe_normal(i * 8 + 2 * e + 1, 7));
     ((FSW_LDS u32x4*)smem)[i] = v;
   }
   __syncthreads();
@@ -79,6 +84,22 @@ __global__ __launch_bounds__(512) void probe_mfma_mix_kernel(const char* src, un
     for (int x = 0; x < 4; x++) {
 #pragma unroll
       for (int q = 0; q < 8; q++) acc[x][q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[x], a[q], acc[x][q], 0, 0, 0);
+      if constexpr (GATING) {
+        // in the same scheduling region as the 8 MFMAs above, so the compiler may put it into their shadow
+        const int nx = (x + 1) & 3;
+        u32x4 w;
+#pragma unroll
+        for (int e = 0; e < 2; e++) {
+          const unsigned d = pending[nx][0][e], g = pending[nx][1][e], u = pending[nx][2][e];
+          float dU0, dG0, dU1, dG1;
+          gating_grad(__uint_as_float(d << 16), __uint_as_float(g << 16), __uint_as_float(u << 16), dU0, dG0);
+          gating_grad(__uint_as_float(d & 0xffff0000u), __uint_as_float(g & 0xffff0000u),
+                      __uint_as_float(u & 0xffff0000u), dU1, dG1);
+          w[e] = BF16::pack2(dG0 * 0.015625f, dG1 * 0.015625f);
+          w[2 + e] = BF16::pack2(dU0 * 0.015625f, dU1 * 0.015625f);
+        }
+        b[nx] = __builtin_bit_cast(bf16x8, w);
+      }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int r = 0; r < NR; r++) {
@@ -166,6 +187,7 @@ int fsw_probe_mfma_mix(int mix, int iters, int workgroups, const void* buf, int6
     case 2: fsw::probe_mfma_mix_kernel<2, 1><<<workgroups, 512, 0, s>>>(src, n, (float*)sink4, iters); break;
     case 3: fsw::probe_mfma_mix_kernel<3, 0><<<workgroups, 512, 0, s>>>(src, n, (float*)sink4, iters); break;
     case 4: fsw::probe_mfma_mix_kernel<0, 1><<<workgroups, 512, 0, s>>>(src, n, (float*)sink4, iters); break;
+    case 5: fsw::probe_mfma_mix_kernel<3, 1, true><<<workgroups, 512, 0, s>>>(src, n, (float*)sink4, iters); break;
     default: return FSW_ERR_BAD_SHAPE;
   }
   if (flop_out) *flop_out = (double)workgroups * 8.0 * iters * 32.0 * 16384.0;

@@ -31,7 +31,10 @@ extern "C" {
  * fsw_probe_mfma_mix: `workgroups` x 8 waves issue `iters` x 32 16x16x32 bf16 MFMAs on ~N(0,1) operands
  * with, per 8 MFMAs, the data movement of mix 0: none, 1: three 16-byte LDS reads per lane + one 1 KiB
  * direct global->LDS load per wave (what the tiled kernels do), 2: two reads + one load, 3: three reads,
- * 4: one load.  The loads walk `bytes` bytes at buf (a multiple of 256 KiB, >= 1 MiB, < 2 GiB).
+ * 4: one load, 5: mix 1 with the weight-side fragment of each 8 MFMAs FORMED from the three values read (taken as
+ * dout, g, u): four gating gradients per lane and 8 MFMAs, the arithmetic a weight-gradient GEMM would carry in its
+ * operand path if the gating-gradient kernel were folded into it.  The loads walk `bytes` bytes at buf (a multiple of
+ * 256 KiB, >= 1 MiB, < 2 GiB).
  */
 FSW_API int fsw_probe_mfma(int random_operands, int iters, int workgroups, void* sink4, void* stream,
                    double* flop_out);
