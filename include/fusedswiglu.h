@@ -152,7 +152,10 @@ FSW_API int fsw_input_grad(const void* grad_xw_gate, const void* grad_xw_up, con
  * instead of a caller workspace; the call itself allocates and frees nothing.  Small problems whose
  * split reduction needs more than that size are rejected with FSW_ERR_SCRATCH_LIMIT (large problems need no
  * scratch and always pass; the optional tail split of a large problem uses the buffer when it fits and is
- * skipped when it does not).  All calls on one GPU share that GPU's buffer:
+ * skipped when it does not).  Results are bit-identical to fsw_input_grad called with a workspace of
+ * FSW_NOALLOC_SCRATCH_BYTES; fsw_input_grad with a larger workspace may split a tail that this call does not,
+ * and then sums in another order (the last bit of a few results in ten thousand differs, the error does not).
+ * All calls on one GPU share that GPU's buffer:
  * calls that overlap in time on one GPU (different streams or threads) race on it.  The first call
  * on a device looks the buffer's address up; make that call outside graph capture.
  */

@@ -85,6 +85,29 @@ def test_no_alloc_large_problem_needs_no_scratch():
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
 
 
+def test_no_alloc_skips_a_tail_split_that_does_not_fit():
+    # 39 x 9 = 351 output tiles: one full round of 256 and a tail of 95, whose split would take 47.5 MiB of partial
+    # tiles.  With the caller's large workspace fsw_input_grad splits the tail; the built-in 32 MiB do not hold it,
+    # so this call runs the tail unsplit: bit-identical to fsw_input_grad given 32 MiB, and equal to the split
+    # result up to the order of the fp32 sums (same distance from an fp32 product).
+    T, D, I = 9984, 2304, 2608
+    dG, dU, wg, wu = _inputs(T, D, I, torch.float16, 11)
+    split, need = _with_workspace(dG, dU, wg, wu, _abi.DTYPE_FP16)
+    assert need > _abi.NOALLOC_SCRATCH_BYTES, "the case is meant to ask for more than the built-in scratch"
+    got = _no_alloc(dG, dU, wg, wu, _abi.DTYPE_FP16)
+    ws = torch.empty(_abi.NOALLOC_SCRATCH_BYTES, dtype=torch.uint8, device=DEV)
+    same_plan = torch.full((T, D), float("nan"), dtype=torch.float16, device=DEV)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    _abi.check(_abi.lib().fsw_input_grad(_ptr(dG), _ptr(dU), _ptr(wg), _ptr(wu), _ptr(same_plan), T, D, I, I, I, D,
+                                         _ptr(ws), _abi.NOALLOC_SCRATCH_BYTES, _abi.DTYPE_FP16, stream))
+    torch.cuda.synchronize()
+    assert torch.equal(got.view(torch.int16), same_plan.view(torch.int16))
+    ref = dG.float() @ wg.float().t() + dU.float() @ wu.float().t()
+    err = lambda a: float((a.float() - ref).norm() / ref.norm())
+    assert err(got) < 5e-3 and abs(err(got) - err(split)) < 1e-6, (err(got), err(split))
+    assert float((got != split).float().mean()) < 1e-2   # a few last bits, not a different result
+
+
 def test_no_alloc_rejects_problems_beyond_the_built_in_scratch():
     T, D, I = 16384, 256, 2048
     L = _abi.lib()
